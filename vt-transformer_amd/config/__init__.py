@@ -1,8 +1,10 @@
 from .base import ConfigError, LayerSpec, ModelConfig, ModelSpec, PartSpec, ScheduleEntry
 from .registry import architectures, config_from_dict, load_config, register_architecture
 from .qwen2 import Qwen2Config
+from .lisunex import LisunexConfig
 
 register_architecture(Qwen2Config.architecture, Qwen2Config)
+register_architecture(LisunexConfig.architecture, LisunexConfig)
 
 __all__ = ["ConfigError", "LayerSpec", "ModelConfig", "ModelSpec", "PartSpec", "ScheduleEntry",
-           "architectures", "config_from_dict", "load_config", "register_architecture", "Qwen2Config"]
+           "architectures", "config_from_dict", "load_config", "register_architecture", "Qwen2Config", "LisunexConfig"]

@@ -44,7 +44,7 @@ class LayerSpec:
 
     block: PartSpec
     mixer: PartSpec
-    feed_forward: PartSpec
+    feed_forward: Optional[PartSpec]   # None: the layer has no feed-forward (and no norm in front of one)
     norms: Dict[str, PartSpec]
     prefix: str  # tensor-name prefix of this layer, e.g. "model.layers.3."
 
@@ -56,10 +56,14 @@ class ScheduleEntry:
     ``layer`` indexes ``ModelSpec.layers`` (a layer may be named twice: its
     weights are shared, each entry still has a cache of its own).
     ``cache_from`` names an earlier entry of the schedule whose cache this
-    entry reads instead of writing its own (None: own cache)."""
+    entry reads instead of writing its own (None: own cache).
+    ``offset_row``: before this entry runs, row ``offset_row`` of the model's
+    table of stream offsets (``ModelSpec.stream_offsets``) is added to every
+    token of the residual stream (None: nothing is added)."""
 
     layer: int
     cache_from: Optional[int] = None
+    offset_row: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -75,10 +79,17 @@ class ModelSpec:
     max_positions: int
     eos_token_ids: List[int] = field(default_factory=list)
     bos_token_id: Optional[int] = None
+    # a tensor [rows, hidden_size] of vectors that schedule entries add to the stream before they run
+    # (``ScheduleEntry.offset_row``): {"name": tensor name, "rows": number of rows}
+    stream_offsets: Optional[Dict[str, Any]] = None
 
     def validate(self) -> None:
         n = len(self.layers)
         for i, e in enumerate(self.schedule):
+            if e.offset_row is not None:
+                rows = int(self.stream_offsets["rows"]) if self.stream_offsets else 0
+                if not 0 <= e.offset_row < rows:
+                    raise ConfigError(f"schedule[{i}] adds row {e.offset_row} of a table of {rows} stream offsets")
             if not 0 <= e.layer < n:
                 raise ConfigError(f"schedule[{i}] names layer {e.layer}, model has {n} layers")
             if e.cache_from is not None:

@@ -28,8 +28,11 @@ def architectures():
 
 def config_from_dict(d: Dict[str, Any]) -> ModelConfig:
     archs = d.get("architectures")
+    if archs is None and isinstance(d.get("architecture"), str):
+        archs = [d["architecture"]]        # some designs name themselves with one string
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
-        raise ConfigError("config.json: key 'architectures' must be a list holding the architecture's name")
+        raise ConfigError("config.json: key 'architectures' must be a list holding the architecture's name "
+                          "(or 'architecture' the name itself)")
     name = archs[0]
     if name not in _ARCHITECTURES:
         raise ConfigError(f"config.json: architecture '{name}' is not registered (known: {', '.join(architectures())})")

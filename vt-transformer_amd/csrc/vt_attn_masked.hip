@@ -1,0 +1,263 @@
+// Attention over paged keys and values for mixers whose heads the other attention kernels do not take: keys and
+// values of different sizes, part of the head rotated, queries and keys scaled to unit root mean square, scores
+// capped by a tanh, keys masked by a window or by chunks of positions, one gate per head.  Two kernels for prompts
+// and decoding alike, in float32 or with 16-bit queries and pages; scores, softmax and sums are float32 in both.
+//
+//   vt_qk_prepare:  per token, rotate the leading `rot` elements of every query and key head (element i with element
+//                   i + rot/2, angles from a table by position), divide by the head's root mean square if asked,
+//                   write the queries out and keys and values into their pages:
+//                   K [page][kv head][slot][D], V [page][kv head][slot][Dv].
+//   vt_attn_masked: one block per (token, query head); keys are visited in chunks of 256 at absolute key indices
+//                   with a running maximum and sum, so a token's result depends only on its position and the keys,
+//                   not on how its request was cut into steps or what else is in the batch.
+//                   score = cap * tanh(scale * q.k / cap) (cap 0: none); key j is seen from position i if j <= i,
+//                   i - j < window (window 0: no bound) and j >= floor(i / chunk) * chunk (chunk 0: no bound);
+//                   out = softmax(score) V * sigmoid(gate[token][head]) (no gate pointer: no gate).
+#include "vt_common.h"
+#include <math.h>
+
+VT_DEFINE_LAST_ERROR()
+
+// ---------------------------------------------------------------------------
+struct PrepArgs {
+    const void* x;          // [n][ldx]: q heads, k heads, v heads, one after the other, from column 0
+    const float* cos_t;     // [max_pos][rot/2]
+    const float* sin_t;
+    const int* positions;
+    const int* tok_entry;
+    const int* block_table;
+    void* q_out;            // [n][H][D]
+    void* k_pages;
+    void* v_pages;
+    long long ldx;
+    int H, G, D, Dv, rot, max_pos, page_size, max_blocks, num_pages, write_kv, unit_rms;
+    float eps;
+};
+
+template <typename TI, typename TC>
+__global__ __launch_bounds__(256) void qk_prepare_kernel(PrepArgs a) {
+    const int t = blockIdx.x;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    const TI* x = (const TI*)a.x + (size_t)t * a.ldx;
+    const int pos = a.positions[t];
+    const int half = a.rot / 2;
+    const float* c = a.cos_t + (size_t)pos * half;
+    const float* s = a.sin_t + (size_t)pos * half;
+    size_t page_row = 0;
+    bool page_ok = false;
+    if (a.write_kv) {
+        const int blk = pos / a.page_size;
+        const int pg = blk < a.max_blocks ? a.block_table[(size_t)a.tok_entry[t] * a.max_blocks + blk] : -1;
+        page_ok = pg >= 0 && pg < a.num_pages;
+        page_row = (size_t)(page_ok ? pg : 0) * a.G * a.page_size + (pos - blk * a.page_size);
+    }
+    const int units = a.H + (a.write_kv ? 2 * a.G : 0);
+    for (int u = wave; u < units; u += nw) {
+        if (u < a.H + a.G) {
+            // a query or key head: rotate, then scale to unit root mean square
+            const bool is_q = u < a.H;
+            const TI* src = x + (size_t)u * a.D;
+            float vals[4];      // D <= 256: up to four elements per lane
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int d = lane + 64 * i;
+                float v = 0.f;
+                if (d < a.D) {
+                    v = load_f32<TI>(src, d);
+                    if (d < a.rot && pos < a.max_pos) {
+                        const bool low = d < half;
+                        const int p = low ? d : d - half;
+                        const float y = load_f32<TI>(src, low ? d + half : d - half);
+                        v = rotate_pair(c[p], s[p], v, y, low);
+                    }
+                }
+                vals[i] = v;
+                ss += v * v;
+            }
+            float r = 1.f;
+            if (a.unit_rms) {
+                ss = wave_sum(ss);
+                r = 1.0f / sqrtf(ss / (float)a.D + a.eps);
+            }
+            if (is_q) {
+                TC* dst = (TC*)a.q_out + ((size_t)t * a.H + u) * a.D;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = lane + 64 * i;
+                    if (d < a.D) store_f32<TC>(dst, d, vals[i] * r);
+                }
+            } else if (page_ok) {
+                const int g = u - a.H;
+                TC* dst = (TC*)a.k_pages + (page_row + (size_t)g * a.page_size) * a.D;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int d = lane + 64 * i;
+                    if (d < a.D) store_f32<TC>(dst, d, vals[i] * r);
+                }
+            }
+        } else if (page_ok) {
+            const int g = u - a.H - a.G;
+            const TI* src = x + (size_t)(a.H + a.G) * a.D + (size_t)g * a.Dv;
+            TC* dst = (TC*)a.v_pages + (page_row + (size_t)g * a.page_size) * a.Dv;
+            for (int d = lane; d < a.Dv; d += 64) store_f32<TC>(dst, d, load_f32<TI>(src, d));
+        }
+    }
+}
+
+extern "C" int vt_qk_prepare(const void* x, int x_dtype, long long ldx, const float* cos_t, const float* sin_t, int rot,
+                             int max_pos, const int* positions, const int* tok_entry, const int* block_table,
+                             int max_blocks, void* q_out, void* k_pages, void* v_pages, int cache_dtype, int page_size,
+                             int num_pages, int n, int H, int G, int D, int Dv, int write_kv, int unit_rms, float eps,
+                             hipStream_t stream) {
+    VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_qk_prepare: bad heads %d/%d", H, G);
+    VT_REQUIRE(D > 0 && D <= 256 && Dv > 0, "vt_qk_prepare: head sizes %d/%d (keys up to 256)", D, Dv);
+    VT_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= D, "vt_qk_prepare: %d rotated elements of %d", rot, D);
+    VT_REQUIRE(rot == 0 || (cos_t && sin_t && max_pos > 0), "vt_qk_prepare: no table of angles");
+    VT_REQUIRE(ldx >= (long long)(H + (write_kv ? G : 0)) * D + (write_kv ? (long long)G * Dv : 0),
+               "vt_qk_prepare: rows of %lld elements are too short", ldx);
+    VT_REQUIRE(!write_kv || (page_size > 0 && max_blocks > 0 && num_pages > 0 && block_table && k_pages && v_pages),
+               "vt_qk_prepare: bad cache sizes");
+    if (n == 0) return 0;
+    PrepArgs a;
+    a.x = x; a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.tok_entry = tok_entry; a.block_table = block_table;
+    a.q_out = q_out; a.k_pages = k_pages; a.v_pages = v_pages; a.ldx = ldx; a.H = H; a.G = G; a.D = D; a.Dv = Dv; a.rot = rot;
+    a.max_pos = max_pos; a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages; a.write_kv = write_kv;
+    a.unit_rms = unit_rms; a.eps = eps;
+    if (x_dtype == VT_F32 && cache_dtype == VT_F32) qk_prepare_kernel<float, float><<<n, 256, 0, stream>>>(a);
+    else if (x_dtype == VT_F32 && cache_dtype == VT_BF16) qk_prepare_kernel<float, bf16_t><<<n, 256, 0, stream>>>(a);
+    else if (x_dtype == VT_BF16 && cache_dtype == VT_BF16) qk_prepare_kernel<bf16_t, bf16_t><<<n, 256, 0, stream>>>(a);
+    else return vt_fail("vt_qk_prepare: dtypes %d -> %d are not handled", x_dtype, cache_dtype);
+    VT_CHECK_LAUNCH("vt_qk_prepare");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+struct MaskedArgs {
+    const void* q;
+    const void* k_pages;
+    const void* v_pages;
+    const int* positions;
+    const int* tok_entry;
+    const int* block_table;
+    const void* gate;       // gate[t * ldg + h], or null
+    void* out;              // [n][H][Dv]
+    long long ldg;
+    int H, G, D, Dv, page_size, max_blocks, num_pages, window, chunk;
+    float scale, cap;
+};
+
+#define KEYS 256
+
+template <typename TC, typename TG>
+__global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
+    extern __shared__ float smem[];
+    float* qs = smem;             // D
+    float* sp = qs + a.D;         // KEYS
+    float* spart = sp + KEYS;     // KEYS
+    __shared__ float red[16];
+
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int D = a.D, Dv = a.Dv, ps = a.page_size;
+    const int kvh = h / (a.H / a.G);
+    const int pos = a.positions[t];
+    const int* bt = a.block_table + (size_t)a.tok_entry[t] * a.max_blocks;
+    int lo = a.chunk > 0 ? (pos / a.chunk) * a.chunk : 0;
+    if (a.window > 0) lo = max(lo, pos - a.window + 1);
+    const TC* kp = (const TC*)a.k_pages;
+    const TC* vp = (const TC*)a.v_pages;
+
+    for (int d = tid; d < D; d += KEYS) qs[d] = load_f32<TC>((const TC*)a.q, ((size_t)t * a.H + h) * D + d);
+    __syncthreads();
+
+    const int Gv = KEYS / Dv;     // key groups for the weighted sum (Dv <= 256)
+    const int d_own = tid % Dv, g_own = tid / Dv;
+    const bool pv_active = g_own < Gv;
+
+    float m = -INFINITY, l = 0.f, acc = 0.f;
+    for (int c0 = (lo / KEYS) * KEYS; c0 <= pos; c0 += KEYS) {
+        const int j = c0 + tid;
+        const bool valid = j >= lo && j <= pos;
+        float s = -INFINITY;
+        if (valid) {
+            const int blk = j / ps;
+            const int pg = bt[blk];
+            if (pg >= 0 && pg < a.num_pages) {
+                const TC* kr = kp + (((size_t)pg * a.G + kvh) * ps + (j - blk * ps)) * D;
+                float dot = 0.f;
+                for (int d = 0; d < D; ++d) dot = fmaf(qs[d], load_f32<TC>(kr, d), dot);
+                s = dot * a.scale;
+                if (a.cap > 0.f) s = a.cap * tanhf(s / a.cap);
+            } else {
+                s = __int_as_float(0x7fc00000);  // a missing page must show, not pass as a masked key
+            }
+        }
+        const float cmax = block_max(s, red);
+        const float m_new = fmaxf(m, cmax);
+        const float p = valid ? expf(s - m_new) : 0.f;
+        sp[tid] = p;
+        const float csum = block_sum(p, red);  // its barriers also publish sp
+        const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+        l = l * alpha + csum;
+
+        float part = 0.f;
+        if (pv_active) {
+            for (int jj = g_own; jj < KEYS; jj += Gv) {
+                const int jk = c0 + jj;
+                if (jk < lo || jk > pos) continue;
+                const int blk = jk / ps;
+                const int pg = bt[blk];
+                if (pg < 0 || pg >= a.num_pages) continue;
+                part = fmaf(sp[jj], load_f32<TC>(vp, (((size_t)pg * a.G + kvh) * ps + (jk - blk * ps)) * Dv + d_own), part);
+            }
+        }
+        spart[tid] = part;
+        __syncthreads();
+        if (tid < Dv) {
+            float sum = 0.f;
+            for (int g = 0; g < Gv; ++g) sum += spart[g * Dv + tid];
+            acc = acc * alpha + sum;
+        }
+        __syncthreads();
+        m = m_new;
+    }
+    if (tid < Dv) {
+        float o = acc / l;
+        if (a.gate) {
+            const float z = load_f32<TG>((const TG*)a.gate, (size_t)t * a.ldg + h);
+            o *= 1.0f / (1.0f + expf(-z));
+        }
+        store_f32<TC>((TC*)a.out, ((size_t)t * a.H + h) * Dv + tid, o);
+    }
+}
+
+extern "C" int vt_attn_masked(const void* q, const void* k_pages, const void* v_pages, int dtype, const int* positions,
+                              const int* tok_entry, const int* block_table, const void* gate, int gate_dtype,
+                              long long ldg, void* out, int n, int H, int G, int D, int Dv, int page_size,
+                              int max_blocks, int num_pages, int window, int chunk, float scale, float cap,
+                              hipStream_t stream) {
+    VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked: bad heads %d/%d", H, G);
+    VT_REQUIRE(D > 0 && Dv > 0 && Dv <= 256, "vt_attn_masked: head sizes %d/%d (values up to 256)", D, Dv);
+    VT_REQUIRE(page_size > 0 && max_blocks > 0 && num_pages > 0, "vt_attn_masked: bad cache sizes");
+    VT_REQUIRE(H <= 65535, "vt_attn_masked: too many heads (%d)", H);
+    VT_REQUIRE(window >= 0 && chunk >= 0 && cap >= 0.f, "vt_attn_masked: bad mask or cap");
+    if (n == 0) return 0;
+    MaskedArgs a;
+    a.q = q; a.k_pages = k_pages; a.v_pages = v_pages; a.positions = positions; a.tok_entry = tok_entry;
+    a.block_table = block_table; a.gate = gate; a.out = out; a.ldg = ldg; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
+    a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages; a.window = window; a.chunk = chunk;
+    a.scale = scale; a.cap = cap;
+    const size_t shmem = (size_t)(D + 2 * KEYS) * sizeof(float);
+    const dim3 grid(n, H);
+    if (dtype == VT_F32) {
+        VT_REQUIRE(!gate || gate_dtype == VT_F32, "vt_attn_masked: float32 takes float32 gates");
+        attn_masked_kernel<float, float><<<grid, KEYS, shmem, stream>>>(a);
+    } else if (dtype == VT_BF16) {
+        if (gate && gate_dtype == VT_BF16) attn_masked_kernel<bf16_t, bf16_t><<<grid, KEYS, shmem, stream>>>(a);
+        else attn_masked_kernel<bf16_t, float><<<grid, KEYS, shmem, stream>>>(a);
+    } else {
+        return vt_fail("vt_attn_masked: unknown dtype %d", dtype);
+    }
+    VT_CHECK_LAUNCH("vt_attn_masked");
+    return 0;
+}

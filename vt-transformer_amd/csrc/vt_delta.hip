@@ -1,0 +1,300 @@
+// The gated delta rule as a token mixer with per-request state, for prompts and decoding alike.
+//
+// Per head, a matrix state S [D][Dv] in float32 is carried from token to token:
+//     S <- g S;   u = beta (v - S^T k);   S <- S + k u^T;   o = S^T q        (the read-out sees the token's own write)
+// with q and k scaled to unit length (q also by D^-1/2), beta = sigmoid(b) and the decay
+// g = exp(-exp(A_log) softplus(a + dt_bias)), all in float32.  In front of it q, k and v pass a short causal
+// convolution over time per channel and a SiLU; the convolution's last taps - 1 inputs are part of the state.
+//
+//   vt_short_conv:        y[t][c] = silu(sum_j taps[c][j] x[t - (K-1) + j][c]); inputs before a request's first token
+//                         of this step come from its state (zeros at the start of a sequence).
+//   vt_short_conv_carry:  the last K-1 inputs of every request go into its state (after vt_short_conv has read it).
+//   vt_delta_rule:        the recurrence.  A block takes 64 value columns of one (request, head); four lanes share a
+//                         column, each holding a quarter of its D state elements in registers.  Tokens are taken in
+//                         tiles of 16 through LDS; every token is computed by the same instructions in the same
+//                         order whatever the tile, so a result does not depend on how the request was cut into steps.
+//   vt_gated_rmsnorm:     out = o / rms(o) * w * silu(gate), per (token, head).
+#include "vt_common.h"
+#include <math.h>
+
+VT_DEFINE_LAST_ERROR()
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// ---------------------------------------------------------------------------
+struct ConvArgs {
+    const void* x;          // [n][ldx], channels 0..C-1
+    const float* taps;      // [C][K]
+    float* state;           // slot s: state + s * slot_stride, [K-1][C]
+    const int* tok_entry;
+    const int* entry_start; // [entries + 1]
+    const int* slots;
+    void* y;                // [n][C]
+    long long ldx, slot_stride;
+    int C, K, n_entries;
+};
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void short_conv_kernel(ConvArgs a) {
+    const int t = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= a.C) return;
+    const int e = a.tok_entry[t];
+    const int start = a.entry_start[e];
+    const float* st = a.state + (size_t)a.slots[e] * a.slot_stride;
+    const int K = a.K;
+    float acc = 0.f;
+    for (int j = 0; j < K; ++j) {
+        const int tau = t - (K - 1) + j;
+        const float v = tau >= start ? load_f32<TI>((const TI*)a.x, (size_t)tau * a.ldx + c)
+                                     : st[(size_t)(K - 1 + tau - start) * a.C + c];
+        acc = fmaf(a.taps[(size_t)c * K + j], v, acc);
+    }
+    store_f32<TO>((TO*)a.y, (size_t)t * a.C + c, silu_f(acc));
+}
+
+#define CONV_MAX_TAPS 16
+
+template <typename TI>
+__global__ __launch_bounds__(256) void short_conv_carry_kernel(ConvArgs a) {
+    const int e = blockIdx.x;
+    const int c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= a.C) return;
+    const int start = a.entry_start[e], end = a.entry_start[e + 1];
+    float* st = a.state + (size_t)a.slots[e] * a.slot_stride;
+    const int keep = a.K - 1;
+    float v[CONV_MAX_TAPS];
+#pragma unroll
+    for (int i = 0; i < CONV_MAX_TAPS; ++i) {
+        if (i < keep) {
+            const int tau = end - keep + i;
+            v[i] = tau >= start ? load_f32<TI>((const TI*)a.x, (size_t)tau * a.ldx + c)
+                                : st[(size_t)(keep + tau - start) * a.C + c];
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < CONV_MAX_TAPS; ++i)
+        if (i < keep) st[(size_t)i * a.C + c] = v[i];
+}
+
+static int conv_args(ConvArgs& a, const void* x, long long ldx, const float* taps, float* state, long long slot_stride,
+                     const int* tok_entry, const int* entry_start, const int* slots, void* y, int n, int n_entries, int C,
+                     int K, const char* who) {
+    VT_REQUIRE(n >= 0 && n_entries >= 0 && C > 0, "%s: bad sizes", who);
+    VT_REQUIRE(K >= 1 && K <= CONV_MAX_TAPS, "%s: %d taps (1 to %d)", who, K, CONV_MAX_TAPS);
+    VT_REQUIRE(ldx >= C && slot_stride >= (long long)(K - 1) * C, "%s: rows or state slots are too short", who);
+    a.x = x; a.taps = taps; a.state = state; a.tok_entry = tok_entry; a.entry_start = entry_start; a.slots = slots; a.y = y;
+    a.ldx = ldx; a.slot_stride = slot_stride; a.C = C; a.K = K; a.n_entries = n_entries;
+    return 0;
+}
+
+extern "C" int vt_short_conv(const void* x, int x_dtype, long long ldx, const float* taps, float* state,
+                             long long slot_stride, const int* tok_entry, const int* entry_start, const int* slots,
+                             void* y, int y_dtype, int n, int n_entries, int C, int K, hipStream_t stream) {
+    ConvArgs a;
+    if (conv_args(a, x, ldx, taps, state, slot_stride, tok_entry, entry_start, slots, y, n, n_entries, C, K, "vt_short_conv"))
+        return -1;
+    VT_REQUIRE(C <= 65535 * 256, "vt_short_conv: too many channels");
+    if (n == 0) return 0;
+    const dim3 grid(n, (C + 255) / 256);
+    if (x_dtype == VT_F32 && y_dtype == VT_F32) short_conv_kernel<float, float><<<grid, 256, 0, stream>>>(a);
+    else if (x_dtype == VT_F32 && y_dtype == VT_BF16) short_conv_kernel<float, bf16_t><<<grid, 256, 0, stream>>>(a);
+    else if (x_dtype == VT_BF16 && y_dtype == VT_BF16) short_conv_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>(a);
+    else if (x_dtype == VT_BF16 && y_dtype == VT_F32) short_conv_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(a);
+    else return vt_fail("vt_short_conv: dtypes %d -> %d are not handled", x_dtype, y_dtype);
+    VT_CHECK_LAUNCH("vt_short_conv");
+    return 0;
+}
+
+extern "C" int vt_short_conv_carry(const void* x, int x_dtype, long long ldx, float* state, long long slot_stride,
+                                   const int* entry_start, const int* slots, int n_entries, int C, int K,
+                                   hipStream_t stream) {
+    ConvArgs a;
+    if (conv_args(a, x, ldx, nullptr, state, slot_stride, nullptr, entry_start, slots, nullptr, 0, n_entries, C, K,
+                  "vt_short_conv_carry"))
+        return -1;
+    if (n_entries == 0 || K == 1) return 0;
+    VT_REQUIRE(C <= 65535 * 256, "vt_short_conv_carry: too many channels");
+    const dim3 grid(n_entries, (C + 255) / 256);
+    if (x_dtype == VT_F32) short_conv_carry_kernel<float><<<grid, 256, 0, stream>>>(a);
+    else if (x_dtype == VT_BF16) short_conv_carry_kernel<bf16_t><<<grid, 256, 0, stream>>>(a);
+    else return vt_fail("vt_short_conv_carry: unknown dtype %d", x_dtype);
+    VT_CHECK_LAUNCH("vt_short_conv_carry");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+struct DeltaArgs {
+    const void* qkv;        // [n][C]: q (G x D), k (G x D), v (H x Dv), after convolution and SiLU
+    const float* ba;        // [n][2H]: beta logits, then decay logits
+    const float* a_log;     // [H]
+    const float* dt_bias;   // [H]
+    float* state;           // slot s: state + s * slot_stride, [H][D][Dv]
+    const int* entry_start;
+    const int* slots;
+    float* o;               // [n][H][Dv]
+    long long slot_stride;
+    int H, G, D, Dv;
+};
+
+#define DELTA_TILE 16
+#define DELTA_COLS 64
+
+// DS: state elements per lane (a quarter of D, rounded up to a power of two from 8 to 64)
+template <typename TI, int DS>
+__global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
+    constexpr int DP = 4 * DS;                        // D padded
+    __shared__ float qs[DELTA_TILE][DP];
+    __shared__ float ks[DELTA_TILE][DP];
+    __shared__ float vs[DELTA_TILE][DELTA_COLS];
+    __shared__ float beta_s[DELTA_TILE], g_s[DELTA_TILE], rq_s[DELTA_TILE], rk_s[DELTA_TILE];
+
+    const int e = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * DELTA_COLS;
+    const int tid = threadIdx.x;
+    const int r = tid & 3, col = col0 + (tid >> 2);
+    const bool col_ok = col < a.Dv;
+    const int D = a.D, Dv = a.Dv, H = a.H, G = a.G;
+    const int kh = h / (H / G);
+    const int C = 2 * G * D + H * Dv;
+    const int start = a.entry_start[e], end = a.entry_start[e + 1];
+    float* S_mem = a.state + (size_t)a.slots[e] * a.slot_stride + (size_t)h * D * Dv;
+    const TI* x = (const TI*)a.qkv;
+    const float decay_rate = expf(a.a_log[h]);
+    const float bias = a.dt_bias[h];
+    const float q_scale = 1.0f / sqrtf((float)D);
+
+    float S[DS];
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = r * DS + i;
+        S[i] = (col_ok && d < D) ? S_mem[(size_t)d * Dv + col] : 0.f;
+    }
+
+    for (int t0 = start; t0 < end; t0 += DELTA_TILE) {
+        const int nt = min(DELTA_TILE, end - t0);
+        __syncthreads();        // the tile before has been read
+        for (int i = tid; i < DELTA_TILE * DP; i += 256) {
+            const int tt = i / DP, d = i % DP;
+            float qv = 0.f, kv = 0.f;
+            if (tt < nt && d < D) {
+                const size_t row = (size_t)(t0 + tt) * C;
+                qv = load_f32<TI>(x, row + (size_t)kh * D + d);
+                kv = load_f32<TI>(x, row + (size_t)(G + kh) * D + d);
+            }
+            qs[tt][d] = qv;
+            ks[tt][d] = kv;
+        }
+        for (int i = tid; i < DELTA_TILE * DELTA_COLS; i += 256) {
+            const int tt = i / DELTA_COLS, j = i % DELTA_COLS;
+            vs[tt][j] = (tt < nt && col0 + j < Dv)
+                            ? load_f32<TI>(x, (size_t)(t0 + tt) * C + (size_t)2 * G * D + (size_t)h * Dv + col0 + j) : 0.f;
+        }
+        __syncthreads();
+        if (tid < nt) {
+            // lengths of q and k, gate and decay of one token, all in float32, sums in index order
+            float sq = 0.f, sk = 0.f;
+            for (int d = 0; d < D; ++d) {
+                sq = fmaf(qs[tid][d], qs[tid][d], sq);
+                sk = fmaf(ks[tid][d], ks[tid][d], sk);
+            }
+            rq_s[tid] = q_scale / sqrtf(sq + 1e-6f);
+            rk_s[tid] = 1.0f / sqrtf(sk + 1e-6f);
+            const float* ba = a.ba + (size_t)(t0 + tid) * 2 * H;
+            beta_s[tid] = 1.0f / (1.0f + expf(-ba[h]));
+            g_s[tid] = expf(-decay_rate * softplus_f(ba[H + h] + bias));
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float g = g_s[tt], beta = beta_s[tt], rq = rq_s[tt], rk = rk_s[tt];
+            const float* kk = &ks[tt][r * DS];
+            const float* qq = &qs[tt][r * DS];
+            float dot = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                S[i] *= g;
+                dot = fmaf(kk[i] * rk, S[i], dot);
+            }
+            dot += __shfl_xor(dot, 1, 64);
+            dot += __shfl_xor(dot, 2, 64);
+            const float u = beta * (vs[tt][tid >> 2] - dot);
+            float out = 0.f;
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                S[i] = fmaf(kk[i] * rk, u, S[i]);
+                out = fmaf(qq[i] * rq, S[i], out);
+            }
+            out += __shfl_xor(out, 1, 64);
+            out += __shfl_xor(out, 2, 64);
+            if (r == 0 && col_ok) a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = out;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < DS; ++i) {
+        const int d = r * DS + i;
+        if (col_ok && d < D) S_mem[(size_t)d * Dv + col] = S[i];
+    }
+}
+
+extern "C" int vt_delta_rule(const void* qkv, int dtype, const float* ba, const float* a_log, const float* dt_bias,
+                             float* state, long long slot_stride, const int* entry_start, const int* slots, float* o,
+                             int n_entries, int H, int G, int D, int Dv, hipStream_t stream) {
+    VT_REQUIRE(n_entries >= 0 && H > 0 && G > 0 && H % G == 0, "vt_delta_rule: bad heads %d/%d", H, G);
+    VT_REQUIRE(D > 0 && D <= 256 && Dv > 0, "vt_delta_rule: head sizes %d/%d (keys up to 256)", D, Dv);
+    VT_REQUIRE(slot_stride >= (long long)H * D * Dv, "vt_delta_rule: state slots are too short");
+    VT_REQUIRE(H <= 65535, "vt_delta_rule: too many heads (%d)", H);
+    if (n_entries == 0) return 0;
+    DeltaArgs a;
+    a.qkv = qkv; a.ba = ba; a.a_log = a_log; a.dt_bias = dt_bias; a.state = state; a.entry_start = entry_start;
+    a.slots = slots; a.o = o; a.slot_stride = slot_stride; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
+    const dim3 grid(n_entries, H, (Dv + DELTA_COLS - 1) / DELTA_COLS);
+    const int quarter = (D + 3) / 4;
+#define VT_DELTA(TI)                                                                          \
+    do {                                                                                      \
+        if (quarter <= 8) delta_rule_kernel<TI, 8><<<grid, 256, 0, stream>>>(a);              \
+        else if (quarter <= 16) delta_rule_kernel<TI, 16><<<grid, 256, 0, stream>>>(a);       \
+        else if (quarter <= 32) delta_rule_kernel<TI, 32><<<grid, 256, 0, stream>>>(a);       \
+        else delta_rule_kernel<TI, 64><<<grid, 256, 0, stream>>>(a);                          \
+    } while (0)
+    if (dtype == VT_F32) VT_DELTA(float);
+    else if (dtype == VT_BF16) VT_DELTA(bf16_t);
+    else return vt_fail("vt_delta_rule: unknown dtype %d", dtype);
+#undef VT_DELTA
+    VT_CHECK_LAUNCH("vt_delta_rule");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// out[t][h][:] = o[t][h][:] / sqrt(mean(o^2) + eps) * w[:] * silu(gate[t][h][:]); gate[t * ldg + h * Dv + j]
+template <typename TG, typename TO>
+__global__ __launch_bounds__(64) void gated_rmsnorm_kernel(const float* __restrict__ o, const float* __restrict__ w,
+                                                           const TG* __restrict__ gate, long long ldg, TO* __restrict__ out,
+                                                           int H, int Dv, float eps) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* row = o + ((size_t)t * H + h) * Dv;
+    float ss = 0.f;
+    for (int j = lane; j < Dv; j += 64) ss = fmaf(row[j], row[j], ss);
+    ss = wave_sum(ss);
+    const float rinv = 1.0f / sqrtf(ss / (float)Dv + eps);
+    for (int j = lane; j < Dv; j += 64) {
+        const float z = load_f32<TG>(gate, (size_t)t * ldg + (size_t)h * Dv + j);
+        store_f32<TO>(out, ((size_t)t * H + h) * Dv + j, row[j] * rinv * w[j] * silu_f(z));
+    }
+}
+
+extern "C" int vt_gated_rmsnorm(const float* o, const float* w, const void* gate, int gate_dtype, long long ldg, void* out,
+                                int out_dtype, int n, int H, int Dv, float eps, hipStream_t stream) {
+    VT_REQUIRE(n >= 0 && H > 0 && Dv > 0 && H <= 65535, "vt_gated_rmsnorm: bad sizes");
+    VT_REQUIRE(ldg >= (long long)H * Dv, "vt_gated_rmsnorm: gate rows are too short");
+    if (n == 0) return 0;
+    const dim3 grid(n, H);
+    if (gate_dtype == VT_F32 && out_dtype == VT_F32)
+        gated_rmsnorm_kernel<float, float><<<grid, 64, 0, stream>>>(o, w, (const float*)gate, ldg, (float*)out, H, Dv, eps);
+    else if (gate_dtype == VT_F32 && out_dtype == VT_BF16)
+        gated_rmsnorm_kernel<float, bf16_t><<<grid, 64, 0, stream>>>(o, w, (const float*)gate, ldg, (bf16_t*)out, H, Dv, eps);
+    else if (gate_dtype == VT_BF16 && out_dtype == VT_BF16)
+        gated_rmsnorm_kernel<bf16_t, bf16_t><<<grid, 64, 0, stream>>>(o, w, (const bf16_t*)gate, ldg, (bf16_t*)out, H, Dv, eps);
+    else return vt_fail("vt_gated_rmsnorm: dtypes %d -> %d are not handled", gate_dtype, out_dtype);
+    VT_CHECK_LAUNCH("vt_gated_rmsnorm");
+    return 0;
+}

@@ -18,23 +18,23 @@ VT_DEFINE_LAST_ERROR()
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
-                             int hidden, int vocab) {
+                             int hidden, int vocab, float scale) {
     int t = blockIdx.x;
     int id = ids[t];
     bool ok = id >= 0 && id < vocab;
     const T* row = table + (size_t)(ok ? id : 0) * hidden;
     float* o = out + (size_t)t * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = ok ? load_f32<T>(row, i) : __int_as_float(0x7fc00000);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) o[i] = ok ? load_f32<T>(row, i) * scale : __int_as_float(0x7fc00000);
 }
 
 extern "C" int vt_embed(const void* table, int table_dtype, const int* ids, float* out, int n, int hidden, int vocab,
-                        hipStream_t stream) {
+                        float scale, hipStream_t stream) {
     VT_REQUIRE(n >= 0 && hidden > 0 && vocab > 0, "vt_embed: bad sizes n=%d hidden=%d vocab=%d", n, hidden, vocab);
     if (n == 0) return 0;
     if (table_dtype == VT_F32)
-        embed_kernel<float><<<n, 256, 0, stream>>>((const float*)table, ids, out, hidden, vocab);
+        embed_kernel<float><<<n, 256, 0, stream>>>((const float*)table, ids, out, hidden, vocab, scale);
     else if (table_dtype == VT_BF16)
-        embed_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)table, ids, out, hidden, vocab);
+        embed_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)table, ids, out, hidden, vocab, scale);
     else
         return vt_fail("vt_embed: unknown table dtype %d", table_dtype);
     VT_CHECK_LAUNCH("vt_embed");
@@ -197,6 +197,34 @@ extern "C" int vt_residual_add(float* h, const void* delta, int delta_dtype, lon
     else if (delta_dtype == VT_BF16) residual_add_kernel<bf16_t><<<blocks, 256, 0, stream>>>(h, (const bf16_t*)delta, (size_t)n);
     else return vt_fail("vt_residual_add: unknown dtype %d", delta_dtype);
     VT_CHECK_LAUNCH("vt_residual_add");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// h[t, :] += delta[t, :] (if any) + row[:]: one vector added to every token of the stream (fp32 sum)
+// ---------------------------------------------------------------------------
+template <typename TD>
+__global__ void add_row_kernel(float* __restrict__ h, const TD* __restrict__ delta, const float* __restrict__ row,
+                               size_t n, int hidden) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float x = h[i];
+    if (delta) x += load_f32<TD>(delta, i);
+    h[i] = x + row[i % (size_t)hidden];
+}
+
+extern "C" int vt_add_row(float* h, const void* delta, int delta_dtype, const float* row, long long tokens, int hidden,
+                          hipStream_t stream) {
+    VT_REQUIRE(hidden > 0 && tokens >= 0, "vt_add_row: bad sizes %lld x %d", tokens, hidden);
+    long long n = tokens * hidden;
+    if (n <= 0) return 0;
+    unsigned blocks = (unsigned)((n + 255) / 256);
+    if (delta == nullptr || delta_dtype == VT_F32)
+        add_row_kernel<float><<<blocks, 256, 0, stream>>>(h, (const float*)delta, row, (size_t)n, hidden);
+    else if (delta_dtype == VT_BF16)
+        add_row_kernel<bf16_t><<<blocks, 256, 0, stream>>>(h, (const bf16_t*)delta, row, (size_t)n, hidden);
+    else return vt_fail("vt_add_row: unknown dtype %d", delta_dtype);
+    VT_CHECK_LAUNCH("vt_add_row");
     return 0;
 }
 

@@ -94,14 +94,15 @@ def _f(v) -> ctypes.c_float:
 
 
 # ---------------------------------------------------------------------------
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale, the product in float32."""
     n = ids.numel()
     vocab, hidden = table.shape
     _chk(table, "embed.table")
     _chk(ids, "embed.ids", torch.int32)
     _chk(out, "embed.out", torch.float32, (n, hidden))
     _run(load_lib("vt_elementwise", half=_half(table)), "vt_embed", _ptr(table), _i(_code(table)), _ptr(ids), _ptr(out), _i(n), _i(hidden),
-         _i(vocab), _stream())
+         _i(vocab), _f(scale), _stream())
     return out
 
 
@@ -131,6 +132,18 @@ def residual_add(h: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
     _chk(delta, "residual_add.delta", None, h.shape)
     _run(load_lib("vt_elementwise", half=_half(delta)), "vt_residual_add", _ptr(h), _ptr(delta), _i(_code(delta)),
          ctypes.c_longlong(h.numel()), _stream())
+    return h
+
+
+def add_row(h: torch.Tensor, delta: Optional[torch.Tensor], row: torch.Tensor) -> torch.Tensor:
+    """h[t] += delta[t] (if given) + row, for every token t: one vector added to the whole stream."""
+    n, hidden = h.shape
+    _chk(h, "add_row.h", torch.float32)
+    _chk(row, "add_row.row", torch.float32, (hidden,))
+    if delta is not None:
+        _chk(delta, "add_row.delta", None, h.shape)
+    _run(load_lib("vt_elementwise", half=_half(delta)), "vt_add_row", _ptr(h), _ptr(delta),
+         _i(_code(delta) if delta is not None else F32), _ptr(row), ctypes.c_longlong(n), _i(hidden), _stream())
     return h
 
 
@@ -639,6 +652,184 @@ def attention_bf16_decode_fused(qkv: torch.Tensor, cos: Optional[torch.Tensor], 
          _ptr(cos), _ptr(sin), _i(rot), _i(max_pos), _ptr(k_pages), _ptr(v_pages), _ptr(block_table), _ptr(entry_pos0),
          _ptr(dec_params), _i(n), _i(p_max), _ptr(out), _ptr(part_o), _ptr(part_ml), _i(n_heads), _i(n_kv),
          _i(page_size), _i(block_table.shape[1]), _i(num_pages), _i(window), _f(scale), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+# attention with separate key and value sizes, capped scores, chunk or window masks and head gates (vt_attn_masked.hip)
+MASKED_MAX_KEY_DIM = 256
+MASKED_MAX_VALUE_DIM = 256
+
+
+def qk_prepare(x: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
+               tok_entry: torch.Tensor, block_table: Optional[torch.Tensor], q_out: torch.Tensor,
+               k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, key_dim: int,
+               value_dim: int, unit_rms_eps: Optional[float], write_kv: bool = True) -> None:
+    """x [n, >= (H + G) D + G Dv]: query heads, key heads, value heads.  Rotates the leading 2 * cos.shape[1] elements
+    of every query and key head by the tables' angles at `positions`, divides each head by its root mean square
+    (eps inside the root) unless unit_rms_eps is None, writes queries to q_out [n, H * D] and, with write_kv, keys and
+    values into their pages ([page][kv][slot][D] and [page][kv][slot][Dv])."""
+    n = x.shape[0]
+    _chk(x, "qk_prepare.x")
+    need = (n_heads + (n_kv if write_kv else 0)) * key_dim + (n_kv * value_dim if write_kv else 0)
+    if x.dim() != 2 or x.shape[1] < need:
+        raise KernelError(f"qk_prepare.x: shape {tuple(x.shape)}, need {need} columns")
+    _chk(positions, "qk_prepare.positions", torch.int32, (n,))
+    _chk(tok_entry, "qk_prepare.tok_entry", torch.int32, (n,))
+    _chk(q_out, "qk_prepare.q_out", None, (n, n_heads * key_dim))
+    if q_out.dtype != torch.float32 and x.dtype not in (torch.float32, q_out.dtype):
+        raise KernelError(f"qk_prepare: {x.dtype} inputs and {q_out.dtype} queries")
+    if q_out.dtype == torch.float32 and x.dtype != torch.float32:
+        raise KernelError("qk_prepare: float32 queries need float32 inputs")
+    rot = max_pos = 0
+    if cos is not None:
+        _chk(cos, "qk_prepare.cos", torch.float32)
+        _chk(sin, "qk_prepare.sin", torch.float32, cos.shape)
+        max_pos, half = cos.shape
+        rot = 2 * half
+        if rot > key_dim:
+            raise KernelError(f"qk_prepare: {rot} rotated elements in heads of {key_dim}")
+    page_size = num_pages = max_blocks = 0
+    if write_kv:
+        _chk(k_pages, "qk_prepare.k_pages", q_out.dtype)
+        num_pages, kvh, page_size, d = k_pages.shape
+        if (kvh, d) != (n_kv, key_dim):
+            raise KernelError(f"qk_prepare.k_pages: shape {tuple(k_pages.shape)} does not fit kv heads {n_kv} x {key_dim}")
+        _chk(v_pages, "qk_prepare.v_pages", q_out.dtype, (num_pages, n_kv, page_size, value_dim))
+        _chk(block_table, "qk_prepare.block_table", torch.int32)
+        max_blocks = block_table.shape[1]
+    _run(load_lib("vt_attn_masked", half=_half(x, q_out)), "vt_qk_prepare", _ptr(x), _i(_code(x)),
+         ctypes.c_longlong(x.stride(0)), _ptr(cos), _ptr(sin), _i(rot), _i(max_pos), _ptr(positions), _ptr(tok_entry),
+         _ptr(block_table), _i(max_blocks), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _i(_code(q_out)), _i(page_size),
+         _i(num_pages), _i(n), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(1 if write_kv else 0),
+         _i(0 if unit_rms_eps is None else 1), _f(unit_rms_eps or 0.0), _stream())
+
+
+def attention_masked(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, positions: torch.Tensor,
+                     tok_entry: torch.Tensor, block_table: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int,
+                     key_dim: int, value_dim: int, scale: float, cap: float = 0.0, window: int = 0, chunk: int = 0,
+                     gate: Optional[torch.Tensor] = None, gate_column: int = 0) -> torch.Tensor:
+    """out [n, H * Dv] = softmax over the seen keys of cap * tanh(scale q.k / cap) (cap 0: scale q.k), times V, times
+    sigmoid(gate[:, gate_column + head]) if `gate` (a 2-d tensor whose rows are the tokens') is given.  Key j is seen
+    from position i if j <= i, i - j < window (0: unbounded) and j is in i's chunk of `chunk` positions (0: unbounded)."""
+    n = q.shape[0]
+    num_pages, kvh, page_size, d = k_pages.shape
+    dt = q.dtype
+    _chk(q, "attention_masked.q", None, (n, n_heads * key_dim))
+    _chk(k_pages, "attention_masked.k_pages", dt, (num_pages, n_kv, page_size, key_dim))
+    _chk(v_pages, "attention_masked.v_pages", dt, (num_pages, n_kv, page_size, value_dim))
+    _chk(out, "attention_masked.out", dt, (n, n_heads * value_dim))
+    _chk(positions, "attention_masked.positions", torch.int32, (n,))
+    _chk(tok_entry, "attention_masked.tok_entry", torch.int32, (n,))
+    _chk(block_table, "attention_masked.block_table", torch.int32)
+    if value_dim > MASKED_MAX_VALUE_DIM:
+        raise KernelError(f"attention_masked: value heads of {value_dim} (up to {MASKED_MAX_VALUE_DIM})")
+    gptr, gcode, ldg = ctypes.c_void_p(0), F32, 0
+    if gate is not None:
+        _chk(gate, "attention_masked.gate")
+        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads:
+            raise KernelError(f"attention_masked.gate: shape {tuple(gate.shape)} has no {n_heads} columns from {gate_column}")
+        if dt == torch.float32 and gate.dtype != torch.float32:
+            raise KernelError("attention_masked: float32 attention takes float32 gates")
+        gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
+        gcode, ldg = _code(gate), gate.stride(0)
+    _run(load_lib("vt_attn_masked", half=_half(q, gate)), "vt_attn_masked", _ptr(q), _ptr(k_pages), _ptr(v_pages), _i(_code(q)),
+         _ptr(positions), _ptr(tok_entry), _ptr(block_table), gptr, _i(gcode), ctypes.c_longlong(ldg), _ptr(out), _i(n),
+         _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size), _i(block_table.shape[1]), _i(num_pages),
+         _i(window), _i(chunk), _f(scale), _f(cap), _stream())
+    return out
+
+
+# ---------------------------------------------------------------------------
+# the gated delta rule and what stands around it (vt_delta.hip)
+DELTA_MAX_KEY_DIM = 256
+CONV_MAX_TAPS = 16
+
+
+def _state_rows(state: torch.Tensor, name: str, need: int):
+    """state [slots, per_slot] float32 (a view whose rows may lie apart): (pointer, stride in floats)."""
+    if not state.is_cuda or state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1:
+        raise KernelError(f"{name}: state must be a float32 [slots, n] tensor on the GPU with unit stride in a slot")
+    if state.shape[1] < need:
+        raise KernelError(f"{name}: state slots of {state.shape[1]} floats, need {need}")
+    return ctypes.c_void_p(state.data_ptr()), ctypes.c_longlong(state.stride(0))
+
+
+def short_conv(x: torch.Tensor, channels: int, taps: torch.Tensor, state: torch.Tensor, tok_entry: torch.Tensor,
+               entry_start: torch.Tensor, slots: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """y[t, c] = silu(sum_j taps[c, j] * x[t - (K-1) + j, c]) for the first `channels` columns of x, causal within
+    each entry of the step; inputs from before the entry's first token are read from state[slot] ([K-1, channels],
+    the oldest first).  The state is not changed (short_conv_carry does that, afterwards)."""
+    n = x.shape[0]
+    _chk(x, "short_conv.x")
+    if x.dim() != 2 or x.shape[1] < channels:
+        raise KernelError(f"short_conv.x: shape {tuple(x.shape)} has no {channels} channels")
+    k = taps.shape[1]
+    _chk(taps, "short_conv.taps", torch.float32, (channels, k))
+    if not 1 <= k <= CONV_MAX_TAPS:
+        raise KernelError(f"short_conv: {k} taps (1 to {CONV_MAX_TAPS})")
+    _chk(y, "short_conv.y", None, (n, channels))
+    _chk(tok_entry, "short_conv.tok_entry", torch.int32, (n,))
+    _chk(entry_start, "short_conv.entry_start", torch.int32)
+    _chk(slots, "short_conv.slots", torch.int32)
+    n_entries = entry_start.numel() - 1
+    sp, ss = _state_rows(state, "short_conv", (k - 1) * channels)
+    _run(load_lib("vt_delta", half=_half(x, y)), "vt_short_conv", _ptr(x), _i(_code(x)), ctypes.c_longlong(x.stride(0)),
+         _ptr(taps), sp, ss, _ptr(tok_entry), _ptr(entry_start), _ptr(slots), _ptr(y), _i(_code(y)), _i(n), _i(n_entries),
+         _i(channels), _i(k), _stream())
+    return y
+
+
+def short_conv_carry(x: torch.Tensor, channels: int, k: int, state: torch.Tensor, entry_start: torch.Tensor,
+                     slots: torch.Tensor) -> None:
+    """state[slot] <- the last k - 1 inputs of every entry (older ones move up where an entry brought fewer)."""
+    _chk(x, "short_conv_carry.x")
+    _chk(entry_start, "short_conv_carry.entry_start", torch.int32)
+    _chk(slots, "short_conv_carry.slots", torch.int32)
+    if x.dim() != 2 or x.shape[1] < channels or not 1 <= k <= CONV_MAX_TAPS:
+        raise KernelError(f"short_conv_carry: x of shape {tuple(x.shape)}, {channels} channels, {k} taps")
+    sp, ss = _state_rows(state, "short_conv_carry", (k - 1) * channels)
+    _run(load_lib("vt_delta", half=_half(x)), "vt_short_conv_carry", _ptr(x), _i(_code(x)), ctypes.c_longlong(x.stride(0)),
+         sp, ss, _ptr(entry_start), _ptr(slots), _i(entry_start.numel() - 1), _i(channels), _i(k), _stream())
+
+
+def delta_rule(qkv: torch.Tensor, ba: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor,
+               entry_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, key_dim: int,
+               value_dim: int) -> torch.Tensor:
+    """The gated delta rule over the tokens of every entry, from and into state[slot] ([H, D, Dv] float32).
+    qkv [n, 2 G D + H Dv]: queries, keys (G heads of D), values (H heads of Dv); ba [n, 2 H] float32: logits of the
+    write strength and of the decay.  out [n, H * Dv] float32."""
+    n = qkv.shape[0]
+    c = 2 * n_kv * key_dim + n_heads * value_dim
+    _chk(qkv, "delta_rule.qkv", None, (n, c))
+    _chk(ba, "delta_rule.ba", torch.float32, (n, 2 * n_heads))
+    _chk(a_log, "delta_rule.a_log", torch.float32, (n_heads,))
+    _chk(dt_bias, "delta_rule.dt_bias", torch.float32, (n_heads,))
+    _chk(out, "delta_rule.out", torch.float32, (n, n_heads * value_dim))
+    _chk(entry_start, "delta_rule.entry_start", torch.int32)
+    _chk(slots, "delta_rule.slots", torch.int32)
+    if key_dim > DELTA_MAX_KEY_DIM or n_heads % n_kv:
+        raise KernelError(f"delta_rule: heads {n_heads}/{n_kv} of {key_dim}")
+    sp, ss = _state_rows(state, "delta_rule", n_heads * key_dim * value_dim)
+    _run(load_lib("vt_delta", half=_half(qkv)), "vt_delta_rule", _ptr(qkv), _i(_code(qkv)), _ptr(ba), _ptr(a_log), _ptr(dt_bias),
+         sp, ss, _ptr(entry_start), _ptr(slots), _ptr(out), _i(entry_start.numel() - 1), _i(n_heads), _i(n_kv),
+         _i(key_dim), _i(value_dim), _stream())
+    return out
+
+
+def gated_rmsnorm(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, gate_column: int, out: torch.Tensor,
+                  n_heads: int, value_dim: int, eps: float) -> torch.Tensor:
+    """out[t, h] = o[t, h] / sqrt(mean(o[t, h]^2) + eps) * weight * silu(gate[t, gate_column + h * Dv ...]), per head."""
+    n = o.shape[0]
+    _chk(o, "gated_rmsnorm.o", torch.float32, (n, n_heads * value_dim))
+    _chk(weight, "gated_rmsnorm.weight", torch.float32, (value_dim,))
+    _chk(gate, "gated_rmsnorm.gate")
+    _chk(out, "gated_rmsnorm.out", None, (n, n_heads * value_dim))
+    if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads * value_dim:
+        raise KernelError(f"gated_rmsnorm.gate: shape {tuple(gate.shape)} has no {n_heads * value_dim} columns from {gate_column}")
+    gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
+    _run(load_lib("vt_delta", half=_half(gate, out)), "vt_gated_rmsnorm", _ptr(o), _ptr(weight), gptr, _i(_code(gate)),
+         ctypes.c_longlong(gate.stride(0)), _ptr(out), _i(_code(out)), _i(n), _i(n_heads), _i(value_dim), _f(eps), _stream())
     return out
 
 

@@ -13,6 +13,7 @@ from typing import Callable, Dict, List, Optional
 import torch
 
 from ..config.base import LayerSpec, ModelSpec, PartSpec
+from ..kernels import ops
 from ..parts.base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, NormedInput, Part, Registry,
                           Runtime, TensorDecl)
 
@@ -35,12 +36,17 @@ class DecoderModel:
         self.final_norm = build_part(NORMS, spec.final_norm, "", rt=rt, width=width)
         self.head = HEADS.build(spec.head, rt=rt, width=width, vocab_size=spec.vocab_size)
         self.schedule = list(spec.schedule)
+        # vectors that schedule entries add to the whole stream before they run (a repeated run of layers tells its
+        # passes apart by them)
+        self.offsets_name: Optional[str] = spec.stream_offsets["name"] if spec.stream_offsets else None
+        self.offsets_rows = int(spec.stream_offsets["rows"]) if spec.stream_offsets else 0
+        self.offsets: Optional[torch.Tensor] = None
 
     def _build_layer(self, ls: LayerSpec, shared: dict):
         rt, width = self.rt, self.spec.hidden_size
         norms = {role: build_part(NORMS, ns, ls.prefix, rt=rt, width=width) for role, ns in ls.norms.items()}
         mixer = build_part(MIXERS, ls.mixer, ls.prefix, rt=rt, width=width, shared=shared)
-        ffn = build_part(FEED_FORWARDS, ls.feed_forward, ls.prefix, rt=rt, width=width)
+        ffn = build_part(FEED_FORWARDS, ls.feed_forward, ls.prefix, rt=rt, width=width) if ls.feed_forward is not None else None
         return BLOCKS.build(ls.block, rt=rt, norms=norms, mixer=mixer, feed_forward=ffn)
 
     # ------------------------------------------------------------------
@@ -59,6 +65,8 @@ class DecoderModel:
                     raise ValueError(f"tensor '{name}' is declared twice with shapes {out[name].shape} and {decl.shape}")
                 if name not in out or not decl.optional:
                     out[name] = decl
+        if self.offsets_name:
+            out[self.offsets_name] = TensorDecl((self.offsets_rows, self.spec.hidden_size), "bias")
         return out
 
     def load(self, get: Callable[[str], torch.Tensor]) -> None:
@@ -67,6 +75,8 @@ class DecoderModel:
             for p in layer.parts():
                 p.load(get, self.rt)
         self.final_norm.load(get, self.rt)
+        if self.offsets_name:
+            self.offsets = self.rt.place(get(self.offsets_name), "bias")
         # a head's loader takes `shared`: tensors by name that other parts have already placed on the device (the
         # embedding's table, which a tied head multiplies by)
         shared = {}
@@ -83,9 +93,16 @@ class DecoderModel:
         last = len(self.schedule) - 1
         for i, entry in enumerate(self.schedule):
             block = self.layers[entry.layer]
+            if entry.offset_row is not None:
+                # what is still to be added goes in with the offset, in one pass over the stream
+                ops.add_row(h, delta if isinstance(delta, torch.Tensor) else None, self.offsets[entry.offset_row])
+                delta = None
             if getattr(block, "takes_next_norm", False):
-                # the norm that the layer behind starts with, which this layer's last product may prepare
-                nxt = getattr(self.layers[self.schedule[i + 1].layer], "first_norm", None) if i < last else None
+                # the norm that the layer behind starts with, which this layer's last product may prepare (not if
+                # the stream still changes in between)
+                behind = self.schedule[i + 1] if i < last else None
+                nxt = (getattr(self.layers[behind.layer], "first_norm", None)
+                       if behind is not None and behind.offset_row is None else None)
                 h, delta = block.forward(h, delta, ctx, caches[i], states[i], next_norm=nxt)
             else:
                 if isinstance(delta, NormedInput):

@@ -34,11 +34,14 @@ class PreNormBlock(Part):
     def __init__(self, *, rt: Runtime, norms, mixer, feed_forward):
         self.rt = rt
         self.norm_in = norms["input"]
-        self.norm_post = norms["post_mixer"]
         self.mixer = mixer
+        # a layer without a feed-forward has only the first sublayer (and no second norm)
         self.feed_forward = feed_forward
+        self.norm_post = norms["post_mixer"] if feed_forward is not None else None
 
     def parts(self):
+        if self.feed_forward is None:
+            return [self.norm_in, self.mixer]
         return [self.norm_in, self.mixer, self.norm_post, self.feed_forward]
 
     @property
@@ -50,6 +53,8 @@ class PreNormBlock(Part):
         """delta: what is still to be added to h (a tensor), None, or this layer's first norm as the layer in front
         has prepared it (a NormedInput; its addition is done).  Returns (h, delta) in the same terms."""
         fuse = can_fuse(self.rt, h.shape[0]) and h.shape[1] % 8 == 0
+        if self.feed_forward is None:
+            return h, self._run(self.mixer, self.norm_in, h, delta, fuse, next_norm, ctx, cache, state)
         y = self._run(self.mixer, self.norm_in, h, delta, fuse, self.norm_post, ctx, cache, state)
         z = self._run(self.feed_forward, self.norm_post, h, y, fuse, next_norm, ctx)
         return h, z

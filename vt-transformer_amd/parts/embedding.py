@@ -21,8 +21,10 @@ from .linear import SKINNY_MAX_ROWS
 class TokenEmbedding(Part):
     replayable = True
 
-    def __init__(self, *, rt: Runtime, width: int, vocab_size: int, name: str):
+    def __init__(self, *, rt: Runtime, width: int, vocab_size: int, name: str, scale: float = 1.0):
+        """scale: a constant that every row is multiplied by on its way into the float32 stream."""
         self.rt, self.width, self.vocab, self.name = rt, int(width), int(vocab_size), name
+        self.scale = float(scale)
         self.table: Optional[torch.Tensor] = None
 
     def tensors(self) -> Dict[str, TensorDecl]:
@@ -33,7 +35,7 @@ class TokenEmbedding(Part):
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
         h = self.rt.buffer("h", (ids.numel(), self.width), torch.float32)
-        return ops.embed(self.table, ids, h)
+        return ops.embed(self.table, ids, h, self.scale)
 
 
 @HEADS.register("linear_head")

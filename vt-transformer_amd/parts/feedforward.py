@@ -25,7 +25,9 @@ class GatedMLP(Part):
     replayable = True
 
     def __init__(self, *, rt: Runtime, width: int, prefix: str, intermediate_size: int, activation: str = "silu",
-                 names: Optional[Dict[str, str]] = None):
+                 names: Optional[Dict[str, str]] = None, weight_suffix: str = ".weight"):
+        """names: the three matrices' names behind the prefix; weight_suffix: what follows a matrix's name in its
+        tensor's name ("" where the tensor is called as the matrix)."""
         if activation != "silu":
             raise ValueError(f"activation '{activation}' is not supported (only 'silu')")
         self.rt = rt
@@ -34,21 +36,22 @@ class GatedMLP(Part):
         n = {"gate": "gate_proj", "up": "up_proj", "down": "down_proj"}
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
+        self.suffix = weight_suffix
         self.w_gu = self.w_down = self.p_gu = self.p_down = None
 
     def tensors(self) -> Dict[str, TensorDecl]:
         nm = self.names
         return {
-            nm["gate"] + ".weight": TensorDecl((self.inter, self.width), "matrix"),
-            nm["up"] + ".weight": TensorDecl((self.inter, self.width), "matrix"),
-            nm["down"] + ".weight": TensorDecl((self.width, self.inter), "matrix"),
+            nm["gate"] + self.suffix: TensorDecl((self.inter, self.width), "matrix"),
+            nm["up"] + self.suffix: TensorDecl((self.inter, self.width), "matrix"),
+            nm["down"] + self.suffix: TensorDecl((self.width, self.inter), "matrix"),
         }
 
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
         nm = self.names
-        self.w_gu = torch.cat([rt.place(get(nm["gate"] + ".weight"), "matrix"),
-                               rt.place(get(nm["up"] + ".weight"), "matrix")], dim=0).contiguous()
-        self.w_down = rt.place(get(nm["down"] + ".weight"), "matrix")
+        self.w_gu = torch.cat([rt.place(get(nm["gate"] + self.suffix), "matrix"),
+                               rt.place(get(nm["up"] + self.suffix), "matrix")], dim=0).contiguous()
+        self.w_down = rt.place(get(nm["down"] + self.suffix), "matrix")
         self.p_gu, self.p_down = rt.pack(self.w_gu, halves=2), rt.pack(self.w_down)
         self.w_gu, self.w_down = rt.row_major(self.w_gu, self.p_gu), rt.row_major(self.w_down, self.p_down)
 

@@ -1,0 +1,138 @@
+"""Attention mixer for heads that `PagedAttention`'s kernels do not take: keys
+and values of different sizes, rotation of part of the head, queries and
+keys scaled to unit root mean square, scores capped by a tanh, keys masked by
+a window or by chunks of positions, and one sigmoid gate per head on the
+output.  Every one of these is a constructor parameter that can be left out.
+
+Per token: q, k, v (and the gates' logits) in one matrix product with the
+biases; rotation, unit scaling and the write into the pages in one kernel;
+scores, cap, mask, float32 softmax, weighted sum and gate in one kernel that
+reads the pages; output projection.
+
+    score(i, j) = cap * tanh(scale * q_i . k_j / cap)                 (cap 0: scale * q_i . k_j)
+    j is seen from i  <=>  j <= i,  i - j < window (if window > 0),  floor(j / chunk) = floor(i / chunk) (if chunk > 0)
+    out_i[h] = sigmoid(gate_i[h]) * sum_j softmax_j(score(i, j)) v_j
+
+Chunks are counted from position 0 of the sequence.  A key that no later
+position can see is dead for the cache manager: the pages' window is the
+mask's reach.
+"""
+from __future__ import annotations
+
+import math
+from typing import Callable, Dict, Optional
+
+import torch
+
+from ..config.base import PartSpec
+from ..kernels import ops
+from .base import MIXERS, POSITIONS, CacheNeed, PageTensor, Part, Runtime, StateNeed, TensorDecl
+from .linear import linear
+
+
+@MIXERS.register("masked_attention")
+class MaskedAttention(Part):
+    replayable = False      # (its launches' grids follow the step's tokens only, but nobody has replayed it yet)
+
+    def __init__(self, *, rt: Runtime, width: int, prefix: str, num_heads: int, num_kv_heads: int, key_dim: int,
+                 value_dim: Optional[int] = None, qkv_bias: bool = False, position: Optional[PartSpec] = None,
+                 scale: Optional[float] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0,
+                 unit_rms_eps: Optional[float] = None, head_gate: bool = False, shared: Optional[dict] = None,
+                 names: Optional[Dict[str, str]] = None):
+        """key_dim / value_dim: sizes of a head's queries and keys / of its values (default: the same);
+        position: a rotary encoding whose `dim` may be smaller than key_dim (the rest of a head passes unchanged);
+        unit_rms_eps: queries and keys are divided by their root mean square per head after the rotation, with
+        this eps inside the root (None: they are not); head_gate: one sigmoid gate per head from a projection of
+        the mixer's input; names: tensor names behind the prefix for q, k, v, o, g and the biases q_bias, k_bias,
+        v_bias."""
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
+        self.rt, self.width = rt, int(width)
+        self.nh, self.nkv, self.d = int(num_heads), int(num_kv_heads), int(key_dim)
+        self.dv = int(value_dim) if value_dim is not None else self.d
+        if not 1 <= self.d <= ops.MASKED_MAX_KEY_DIM or not 1 <= self.dv <= ops.MASKED_MAX_VALUE_DIM:
+            raise ValueError(f"head sizes {self.d}/{self.dv}: the kernels take keys up to {ops.MASKED_MAX_KEY_DIM} and "
+                             f"values up to {ops.MASKED_MAX_VALUE_DIM}")
+        self.qkv_bias, self.head_gate = bool(qkv_bias), bool(head_gate)
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
+        self.softcap, self.window, self.chunk = float(softcap), int(window), int(chunk)
+        if self.softcap < 0 or self.window < 0 or self.chunk < 0:
+            raise ValueError("softcap, window and chunk must not be negative (0 switches each off)")
+        self.unit_rms_eps = None if unit_rms_eps is None else float(unit_rms_eps)
+        n = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "g": "g_proj.weight",
+             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias"}
+        n.update(names or {})
+        self.names = {k: prefix + v for k, v in n.items()}
+        pos_spec = position or PartSpec("none", {})
+        shared = shared if shared is not None else {}
+        key = "position:" + pos_spec.key()
+        if key not in shared:
+            shared[key] = POSITIONS.build(pos_spec, rt=rt)
+        self.position = shared[key]
+        if getattr(self.position, "dim", 0) > self.d:
+            raise ValueError(f"{self.position.dim} rotated elements in heads of {self.d}")
+        if getattr(self.position, "dim", 0) and not hasattr(self.position, "rotary_tables"):
+            raise ValueError("this mixer takes rotary position encodings (or none)")
+        self.w_in = self.b_in = self.b_in_lowp = self.p_in = self.w_o = self.p_o = None
+
+    # columns of the input projection: queries, keys, values, gates
+    @property
+    def _gate_column(self) -> int:
+        return (self.nh + self.nkv) * self.d + self.nkv * self.dv
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        """Keys [kv head][slot][D] and values [kv head][slot][Dv] in the runtime's dtype.  The mask's reach bounds how
+        long a key lives: with chunks, a key is never seen from `chunk` or more positions later."""
+        reach = [w for w in (self.window, self.chunk) if w > 0]
+        return CacheNeed((PageTensor("k", (self.nkv, self.d), slot_axis=1), PageTensor("v", (self.nkv, self.dv), slot_axis=1)),
+                         window=min(reach) if reach else 0, page_multiple=1)
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def tensors(self) -> Dict[str, TensorDecl]:
+        nm = self.names
+        t = {
+            nm["q"]: TensorDecl((self.nh * self.d, self.width), "matrix"),
+            nm["k"]: TensorDecl((self.nkv * self.d, self.width), "matrix"),
+            nm["v"]: TensorDecl((self.nkv * self.dv, self.width), "matrix"),
+            nm["o"]: TensorDecl((self.width, self.nh * self.dv), "matrix"),
+        }
+        if self.qkv_bias:
+            t[nm["q_bias"]] = TensorDecl((self.nh * self.d,), "bias")
+            t[nm["k_bias"]] = TensorDecl((self.nkv * self.d,), "bias")
+            t[nm["v_bias"]] = TensorDecl((self.nkv * self.dv,), "bias")
+        if self.head_gate:
+            t[nm["g"]] = TensorDecl((self.nh, self.width), "matrix")
+        return t
+
+    def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
+        nm = self.names
+        mats = [rt.place(get(nm[k]), "matrix") for k in (("q", "k", "v", "g") if self.head_gate else ("q", "k", "v"))]
+        self.w_in = torch.cat(mats, dim=0).contiguous()
+        if self.qkv_bias:
+            b = [rt.place(get(nm[k]), "bias") for k in ("q_bias", "k_bias", "v_bias")]
+            if self.head_gate:
+                b.append(torch.zeros(self.nh, dtype=torch.float32, device=rt.device))
+            self.b_in = torch.cat(b, dim=0).contiguous()
+            self.b_in_lowp = self.b_in.to(rt.dtype)
+        self.w_o = rt.place(get(nm["o"]), "matrix")
+        self.p_in, self.p_o = rt.pack(self.w_in), rt.pack(self.w_o)
+        self.w_in, self.w_o = rt.row_major(self.w_in, self.p_in), rt.row_major(self.w_o, self.p_o)
+
+    def forward(self, x, ctx, cache, state=None):
+        rt, nh, nkv, d, dv = self.rt, self.nh, self.nkv, self.d, self.dv
+        n = x.shape[0]
+        if not cache.writes:
+            raise RuntimeError("this mixer does not read another layer's keys and values")
+        y = linear(rt, x, self.w_in, self.b_in, "mattn.in", bias_lowp=self.b_in_lowp, packed=self.p_in)
+        tables = self.position.rotary_tables(ctx.n_positions) if getattr(self.position, "dim", 0) else None
+        cos, sin = tables if tables is not None else (None, None)
+        q = rt.buffer("mattn.q", (n, nh * d), rt.dtype)
+        ops.qk_prepare(y, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, nkv,
+                       d, dv, self.unit_rms_eps)
+        out = rt.buffer("mattn.out", (n, nh * dv), rt.dtype)
+        ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
+                             dv, self.scale, self.softcap, self.window, self.chunk,
+                             gate=y if self.head_gate else None, gate_column=self._gate_column)
+        return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o)
