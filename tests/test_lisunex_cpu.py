@@ -1,0 +1,100 @@
+"""Lisunex without a GPU: its configuration (keys, run order, tensors, errors) and the plain implementation's
+mechanisms against cases whose answers are known."""
+import copy
+import math
+
+import pytest
+import torch
+
+import plain_lisunex as pl
+from lisunex_helpers import CONFIGS, attention_layer, delta_layer, make_weights
+from vt_transformer_amd.config import ConfigError, config_from_dict
+from vt_transformer_amd.weights.random_init import declared_tensors
+
+
+def test_run_order_and_offsets():
+    spec = config_from_dict(copy.deepcopy(CONFIGS["A"])).to_spec()
+    assert [(e.layer, e.offset_row) for e in spec.schedule] == [(0, 0), (1, None), (0, 1), (1, None), (0, 2), (1, None), (2, None)]
+    assert spec.stream_offsets == {"name": "loop.step", "rows": 3}
+    assert pl.layer_runs(CONFIGS["A"]) == [(e.layer, e.offset_row) for e in spec.schedule]
+    spec = config_from_dict(copy.deepcopy(CONFIGS["B"])).to_spec()
+    assert [(e.layer, e.offset_row) for e in spec.schedule] == [(i, None) for i in range(4)] and spec.stream_offsets is None
+    spec = config_from_dict(copy.deepcopy(CONFIGS["C"])).to_spec()
+    assert [(e.layer, e.offset_row) for e in spec.schedule] == [(0, None), (1, 0), (2, None)]
+
+
+def test_parts_and_tensors_follow_the_configuration():
+    cfg = config_from_dict(copy.deepcopy(CONFIGS["A"]))
+    spec = cfg.to_spec()
+    assert [ls.mixer.kind for ls in spec.layers] == ["gated_delta", "masked_attention", "gated_delta"]
+    assert [ls.feed_forward is not None for ls in spec.layers] == [True, False, False]
+    att = spec.layers[1].mixer.params
+    assert (att["key_dim"], att["value_dim"], att["chunk"], att["softcap"], att["scale"]) == (32, 48, 24, 15.0, 0.2)
+    assert att["position"].params["dim"] == 8 and att["position"].params["scaling"]["factor"] == 4.0
+    t = declared_tensors(cfg)
+    assert t["loop.step"].shape == (3, 96) and t["embed"].shape == (203, 96) and t["head"].shape == (203, 96)
+    assert t["l0.mix.q.conv"].shape == (2 * 16, 3) and t["l0.mix.v.conv"].shape == (4 * 24, 3)
+    assert t["l0.mix.b"].shape == (4, 96) and t["l0.mix.A_log"].shape == (4,) and t["l0.mix.norm"].shape == (24,)
+    assert t["l1.mix.q.b"].shape == (4 * 32,) and t["l1.mix.v"].shape == (2 * 48, 96) and t["l1.mix.g"].shape == (4, 96)
+    assert t["l1.mix.o"].shape == (96, 4 * 48) and "l1.norm2" not in t and "l1.mlp.gate" not in t
+    assert t["l0.mlp.down"].shape == (96, 80) and "l0.norm2" in t
+    assert set(make_weights(CONFIGS["A"], 0)) == set(t)
+    assert config_from_dict(cfg.to_dict()).to_dict() == cfg.to_dict()
+
+
+@pytest.mark.parametrize("change,text", [
+    (lambda c: c["layers"][0].update(type="conv"), "mixer type"),
+    (lambda c: c["layers"][1]["mixer"].update(kv_heads=3), "multiple"),
+    (lambda c: c["layers"][1]["mixer"]["rot"].update(dims=34), "dims"),
+    (lambda c: c["layers"][1]["mixer"].pop("scale"), "scale"),
+    (lambda c: c["loop"].update(stop=9), "loop"),
+    (lambda c: c.pop("norm"), "norm"),
+    (lambda c: c["layers"][0]["mlp"].update(kind="routed"), "kind"),
+])
+def test_configuration_errors(change, text):
+    cfg = copy.deepcopy(CONFIGS["A"])
+    change(cfg)
+    with pytest.raises(ConfigError, match=text):
+        config_from_dict(cfg)
+
+
+def test_plain_delta_rule_on_known_cases():
+    # one token: S = k u^T with u = beta v, so o = beta (k.q) v whatever the decay
+    q, k, v = torch.randn(1, 1, 5, dtype=pl.DT), torch.randn(1, 1, 5, dtype=pl.DT), torch.randn(1, 1, 3, dtype=pl.DT)
+    o = pl.delta_rule(q, k, v, torch.tensor([[0.7]], dtype=pl.DT), torch.tensor([[0.3]], dtype=pl.DT))
+    assert torch.allclose(o[0, 0], 0.7 * (k[0, 0] @ q[0, 0]) * v[0, 0])
+    # beta 1, no decay, the same unit key twice: the second write replaces the first value
+    k2 = torch.tensor([[[1.0, 0.0]], [[1.0, 0.0]]], dtype=pl.DT)
+    v2 = torch.tensor([[[2.0]], [[5.0]]], dtype=pl.DT)
+    o = pl.delta_rule(k2, k2, v2, torch.ones(2, 1, dtype=pl.DT), torch.ones(2, 1, dtype=pl.DT))
+    assert torch.allclose(o[:, 0, 0], torch.tensor([2.0, 5.0], dtype=pl.DT))
+
+
+def test_plain_short_conv_and_chunks():
+    x = torch.arange(1.0, 6.0, dtype=pl.DT)[:, None]
+    y = pl.short_conv(x, torch.tensor([[100.0, 10.0, 1.0]], dtype=pl.DT))       # the last column is the current token's
+    assert y[:, 0].tolist() == [1.0, 12.0, 123.0, 234.0, 345.0]
+    t = 10
+    q, k = torch.zeros(t, 1, 4, dtype=pl.DT), torch.zeros(t, 1, 4, dtype=pl.DT)
+    v = torch.arange(t, dtype=pl.DT).reshape(t, 1, 1)
+    o = pl.chunk_attention(q, k, v, torch.arange(t), 1.0, 0.0, 4)[:, 0, 0]      # equal scores: the mean of the seen values
+    assert torch.allclose(o, torch.tensor([0, .5, 1, 1.5, 4, 4.5, 5, 5.5, 8, 8.5], dtype=pl.DT))
+
+
+def test_plain_frequencies():
+    f, mag = pl.yarn_frequencies(16, 1e4, None)
+    assert mag == 1.0 and torch.allclose(f, torch.pow(torch.tensor(1e4, dtype=pl.DT), -torch.arange(8, dtype=pl.DT) / 8))
+    f2, mag2 = pl.yarn_frequencies(16, 1e4, {"factor": 1.0, "original": 128, "fast": 8.0, "slow": 1.0})
+    assert torch.allclose(f, f2) and mag2 == 1.0
+    f3, mag3 = pl.yarn_frequencies(16, 1e4, {"factor": 8.0, "original": 128, "fast": 8.0, "slow": 1.0})
+    assert f3[0] == f[0] and abs(float(f3[-1] / f[-1]) - 0.125) < 1e-12 and abs(mag3 - (1 + 0.1 * math.log(8))) < 1e-12
+
+
+def test_stretched_frequencies_of_the_rotary_part():
+    from vt_transformer_amd.parts.rotary import rotary_table
+    sc = {"factor": 6.0, "original": 200, "fast": 10.0, "slow": 0.5}
+    cos, sin = rotary_table(64, 12, 777.0, sc)
+    f, mag = pl.yarn_frequencies(12, 777.0, sc)
+    ang = torch.arange(64, dtype=pl.DT)[:, None] * f[None, :]
+    assert float((torch.from_numpy(cos).double() - torch.cos(ang) * mag).abs().max()) < 1e-7
+    assert float((torch.from_numpy(sin).double() - torch.sin(ang) * mag).abs().max()) < 1e-7
