@@ -80,7 +80,7 @@ def make_weights(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:
         elif name == "embed":
             t = torch.randn(shape, generator=g)
         else:
-            t = torch.randn(shape, generator=g) * (1.5 / shape[-1] ** 0.5)
+            t = torch.randn(shape, generator=g) / shape[-1] ** 0.5
         out[name] = t.to(torch.bfloat16)
     return out
 
