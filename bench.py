@@ -170,6 +170,89 @@ class Bench:
         return best, steps, int(sum(int(n) for n in lens))
 
 
+# Sizes at which Lisunex (attention and gated-delta layers in turn, a feed-forward behind each) is measured beside a
+# Qwen2 model of the same width, depth, heads and feed-forward: (width, layers, heads, kv heads, head size, ff, vocab)
+PAIR_SIZES = {"1k": (1024, 8, 8, 2, 128, 4096, 32000), "2k": (2048, 12, 16, 4, 128, 8192, 32000),
+              "4k": (4096, 8, 32, 8, 128, 14336, 32000)}
+
+
+def pair_configs(key: str, chunk: int):
+    """(Lisunex config.json, Qwen2 config.json) of equal sizes."""
+    width, layers, heads, kv, d, ff, vocab = PAIR_SIZES[key]
+    att = {"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+           "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5, "softcap": 50.0,
+                     "mask": {"size": chunk},
+                     "rot": {"dims": d // 2, "base": 1e6, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    delta = {"type": "delta", "mlp": {"kind": "dense", "ff": ff},
+             "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "conv": 4}}
+    lis = {"architecture": "Lisunex", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
+           "layers": [att if i % 2 == 0 else delta for i in range(layers)], "loop": None, "max_positions": 32768}
+    qwen = dict(QWEN2_7B, vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
+                num_attention_heads=heads, num_key_value_heads=kv, head_dim=d, max_position_embeddings=32768)
+    return lis, qwen
+
+
+class PairBench(Bench):
+    """Bench's measurements on an engine built from any config.json."""
+
+    def __init__(self, name: str, cfg_d: dict, dtype: str, max_batch: int, pool_tokens: int, ctx_len: int, graphs: bool = True):
+        import numpy as np
+        import torch
+        from vt_transformer_amd.config import config_from_dict
+        from vt_transformer_amd.engine import Engine
+        self.torch, self.np = torch, np
+        self.model_name, self.single_copy = name, False
+        self.cfg = config_from_dict(cfg_d)
+        self.ctx_len = ctx_len
+        self.rs = np.random.RandomState(0)
+        t0 = time.time()
+        self.eng = Engine(config=self.cfg, random_weights_seed=0, dtype=dtype, page_size=16, num_pages=-(-pool_tokens // 16),
+                          max_running_reqs=max_batch, max_seq_len=ctx_len, max_extend_tokens=8192, chunk_size=2048,
+                          decode_graphs=graphs)
+        torch.cuda.synchronize()
+        print(f"[bench] {name}: model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
+
+
+def lisunex_pairs(args) -> int:
+    """Prefill and decode of Lisunex beside Qwen2 at equal sizes; one JSON line."""
+    keys = [k.strip() for k in args.lisunex.split(",") if k.strip()]
+    for k in keys:
+        if k not in PAIR_SIZES:
+            print(f"bench.py: --lisunex takes {', '.join(PAIR_SIZES)}; got '{k}'")
+            return 2
+    T, batch, prompt_len = args.prefill_tokens, args.batch, args.prompt_len or 1024
+    per_req = -(-(prompt_len + args.steps + args.warmup + 32) // 16) * 16
+    pool = max(batch * per_req, T + 64)
+    out = {}
+    for k in keys:
+        lis, qwen = pair_configs(k, args.lisunex_chunk)
+        row = {}
+        for name, cfg_d in (("lisunex", lis), ("qwen2", qwen)):
+            b = PairBench(f"{name} {k}", cfg_d, args.dtype, batch, pool, max(pool // batch, T + 64) + 64, graphs=not args.no_graphs)
+            p_dt = b.prefill_run(T)
+            tps, ms, _ = b.decode_run(batch, args.steps, args.warmup, prompt_len)
+            row[name] = {"prefill_tok_s": round(T / p_dt, 1), "prefill_ms": round(p_dt * 1e3, 3),
+                         "decode_tok_s": round(tps, 1), "decode_ms_per_step": round(ms, 4)}
+            b.close()
+        row["lisunex_over_qwen2"] = {"prefill": round(row["lisunex"]["prefill_tok_s"] / row["qwen2"]["prefill_tok_s"], 3),
+                                     "decode": round(row["lisunex"]["decode_tok_s"] / row["qwen2"]["decode_tok_s"], 3)}
+        width, layers, heads, kv, d, ff, vocab = PAIR_SIZES[k]
+        row["sizes"] = f"L{layers} H{width} NH{heads} KVH{kv} D{d} I{ff} V{vocab}"
+        out[k] = row
+    first = out[keys[0]]
+    print(json.dumps({
+        "metric": f"Lisunex decode tok/s at batch {batch} after {prompt_len:,}-token prompts, sizes {keys[0]} "
+                  f"(beside Qwen2 at equal sizes; prefill of {T:,} tokens under `pairs`)",
+        "value": first["lisunex"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first["lisunex"]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": {"bfloat16": "bf16", "float16": "fp16"}[args.dtype],
+        "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
+        "config": {"model": "Lisunex and Qwen2 at equal sizes", "global_batch": batch, "seq_len": prompt_len,
+                   "prefill_tokens": T, "chunk": args.lisunex_chunk, "parallelism": "1 GPU"},
+        "pairs": out}), flush=True)
+    return 0
+
+
 def mixed_lengths(n: int, seed: int = 0):
     import numpy as np
     return np.random.RandomState(seed).randint(16, 4097, size=n)
@@ -208,10 +291,20 @@ def main() -> int:
                          "4,096 and --mixed-decode tokens each, through the scheduler (portions of prompts beside "
                          "decoded tokens); value = generated tokens per second from first arrival to last token")
     ap.add_argument("--mixed-decode", type=int, default=256)
+    ap.add_argument("--lisunex", default="", metavar="SIZES",
+                    help="another workload instead: the Lisunex design (attention and gated-delta layers in turn) beside "
+                         "Qwen2 at equal sizes, prefill of --prefill-tokens and decode at --batch; sizes by name, "
+                         "with commas: " + ", ".join(PAIR_SIZES))
+    ap.add_argument("--lisunex-chunk", type=int, default=1024, help="positions per chunk of Lisunex's attention mask")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; N > 1 is not measured")
         return 2
+
+    if args.lisunex:
+        if args.dtype == "float16":
+            args.dtype = "bfloat16"         # the serving dtype of this design
+        return lisunex_pairs(args)
 
     import torch
 

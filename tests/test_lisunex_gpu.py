@@ -103,6 +103,7 @@ def test_embedding_scale_and_stream_offsets():
     (3, 3, 16, 16, 16, 7, 0, 0.0, False, False),     # whole head rotated, nothing else but the chunks
     (6, 1, 40, 24, 0, 0, 0, 5.0, True, True),        # no rotation, every earlier key
     (2, 1, 24, 136, 12, 50, 20, 0.0, True, False),   # window inside chunks, values larger than keys
+    (2, 1, 64, 80, 16, 50, 20, 10.0, True, True),    # the same on the matrix cores (heads in multiples of 16)
 ])
 def test_masked_attention_part(dtype, nh, kvh, d, dv, rot, chunk, window, cap, gate, unit):
     from vt_transformer_amd.engine.step import ModelRunner
@@ -159,8 +160,8 @@ def _one_row(q, k, v, scale, cap):
     return out
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_one_key_that_stands_out_at_chunk_and_page_edges(dtype):
+@pytest.mark.parametrize("dtype,matrix", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+def test_one_key_that_stands_out_at_chunk_and_page_edges(dtype, matrix):
     """Queries and keys are made so that one key far back (hundreds of keys away, the last slot of a page, the last
     position of a chunk) takes nearly all the weight from whoever sees it: the positions just inside its chunk must
     return its value, the first position of the next chunk must not, in a prompt's portion and decoded alone."""
@@ -168,7 +169,7 @@ def test_one_key_that_stands_out_at_chunk_and_page_edges(dtype):
     from vt_transformer_amd.kernels import ops
     from vt_transformer_amd.parts import MIXERS
     rt = runtime(dtype)
-    nh, kvh, d, dv, chunk = 2, 1, 16, 8, 320
+    nh, kvh, d, dv, chunk = 2, 1, 16, 16, 320
     mixer = MIXERS.build(PartSpec("masked_attention", dict(num_heads=nh, num_kv_heads=kvh, key_dim=d, value_dim=dv,
                                                            scale=1.0, chunk=chunk)), rt=rt, width=8, prefix="a.", shared={})
     runner = ModelRunner(OneMixer(mixer), rt, 16, 1024, 2, 1024)
@@ -193,8 +194,12 @@ def test_one_key_that_stands_out_at_chunk_and_page_edges(dtype):
             out = torch.empty(b - a, nh * dv, dtype=dtype, device=DEV)
             ops.qk_prepare(yy, None, None, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, kvh,
                            d, dv, None)
-            ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, kvh, d,
-                                 dv, 1.0, 0.0, 0, chunk)
+            if matrix and b - a > 1:        # (the mixer sends steps of single tokens to the other kernel)
+                ops.attention_masked_mfma(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table,
+                                          ctx.extra[("masked_attention.tiles", 16)], out, nh, kvh, d, dv, 1.0, 0.0, 0, chunk)
+            else:
+                ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, kvh,
+                                     d, dv, 1.0, 0.0, 0, chunk)
             outs.append(out.float().cpu())
             runner.cache.commit("r", b)
         runner.release("r")

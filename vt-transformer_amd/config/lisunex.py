@@ -64,6 +64,10 @@ class LisunexConfig(ModelConfig):
 
     architecture = "Lisunex"
 
+    @property
+    def vocab_size(self) -> int:
+        return self.vocab
+
     @classmethod
     def from_dict(cls, d: Dict[str, Any]) -> "LisunexConfig":
         layers = d.get("layers")

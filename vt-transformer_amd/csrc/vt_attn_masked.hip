@@ -6,7 +6,7 @@
 //   vt_qk_prepare:  per token, rotate the leading `rot` elements of every query and key head (element i with element
 //                   i + rot/2, angles from a table by position), divide by the head's root mean square if asked,
 //                   write the queries out and keys and values into their pages:
-//                   K [page][kv head][slot][D], V [page][kv head][slot][Dv].
+//                   K [page][kv head][slot][D], V [page][kv head][Dv][slot].
 //   vt_attn_masked: one block per (token, query head); keys are visited in chunks of 256 at absolute key indices
 //                   with a running maximum and sum, so a token's result depends only on its position and the keys,
 //                   not on how its request was cut into steps or what else is in the batch.
@@ -44,12 +44,15 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(PrepArgs a) {
     const float* c = a.cos_t + (size_t)pos * half;
     const float* s = a.sin_t + (size_t)pos * half;
     size_t page_row = 0;
+    int page_no = 0, page_slot = 0;
     bool page_ok = false;
     if (a.write_kv) {
         const int blk = pos / a.page_size;
         const int pg = blk < a.max_blocks ? a.block_table[(size_t)a.tok_entry[t] * a.max_blocks + blk] : -1;
         page_ok = pg >= 0 && pg < a.num_pages;
-        page_row = (size_t)(page_ok ? pg : 0) * a.G * a.page_size + (pos - blk * a.page_size);
+        page_no = page_ok ? pg : 0;
+        page_slot = pos - blk * a.page_size;
+        page_row = (size_t)page_no * a.G * a.page_size + page_slot;
     }
     const int units = a.H + (a.write_kv ? 2 * a.G : 0);
     for (int u = wave; u < units; u += nw) {
@@ -97,10 +100,11 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(PrepArgs a) {
                 }
             }
         } else if (page_ok) {
+            // values transposed inside the page, [kv head][Dv][slot]: the matrix-core kernel reads keys four at a time
             const int g = u - a.H - a.G;
             const TI* src = x + (size_t)(a.H + a.G) * a.D + (size_t)g * a.Dv;
-            TC* dst = (TC*)a.v_pages + (page_row + (size_t)g * a.page_size) * a.Dv;
-            for (int d = lane; d < a.Dv; d += 64) store_f32<TC>(dst, d, load_f32<TI>(src, d));
+            TC* dst = (TC*)a.v_pages + ((size_t)page_no * a.G + g) * a.Dv * a.page_size + page_slot;
+            for (int d = lane; d < a.Dv; d += 64) store_f32<TC>(dst, (size_t)d * a.page_size, load_f32<TI>(src, d));
         }
     }
 }
@@ -208,7 +212,7 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
                 const int blk = jk / ps;
                 const int pg = bt[blk];
                 if (pg < 0 || pg >= a.num_pages) continue;
-                part = fmaf(sp[jj], load_f32<TC>(vp, (((size_t)pg * a.G + kvh) * ps + (jk - blk * ps)) * Dv + d_own), part);
+                part = fmaf(sp[jj], load_f32<TC>(vp, (((size_t)pg * a.G + kvh) * Dv + d_own) * ps + (jk - blk * ps)), part);
             }
         }
         spart[tid] = part;

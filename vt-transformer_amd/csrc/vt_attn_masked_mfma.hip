@@ -1,0 +1,179 @@
+// The 16-bit attention of vt_attn_masked.hip on the matrix cores, for steps that bring portions of prompts: capped
+// scores, chunk or window masks, key and value heads of different sizes (both multiples of 16, fixed when this file
+// is compiled: VT_KEY_DIM, VT_VALUE_DIM), one gate per head.
+//
+// A wave takes a tile of up to 16 consecutive tokens of one request and one query head; the host lists the tiles
+// (first row, rows).  Per 16 keys (one page, or part of one: pages hold a multiple of 16 keys):
+//     S^T = K Q^T      [16 keys x 16 queries], v_mfma_f32_16x16x16 over the key size; A = K rows from the page
+//                      ([kv head][slot][D]: a lane reads 4 consecutive elements of its key), B = Q from registers
+//     cap, mask, running maximum and sum per query (a query is a column: its 16 scores lie in 4 lanes x 4 registers)
+//     O^T += V^T P^T   [Dv x 16 queries]; A = V^T from the page ([kv head][Dv][slot]: a lane reads 4 consecutive keys of
+//                      its value element), B = P^T, which is exactly what the lane holds of S^T
+// so the probabilities never leave the registers.  Scores, softmax and sums are float32.
+#include "vt_common.h"
+#include <math.h>
+
+VT_DEFINE_LAST_ERROR()
+
+#ifndef VT_KEY_DIM
+#error "compile with -DVT_KEY_DIM=<multiple of 16> -DVT_VALUE_DIM=<multiple of 16>"
+#endif
+static_assert(VT_KEY_DIM % 16 == 0 && VT_KEY_DIM >= 16 && VT_KEY_DIM <= 256, "key size");
+static_assert(VT_VALUE_DIM % 16 == 0 && VT_VALUE_DIM >= 16 && VT_VALUE_DIM <= 256, "value size");
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+struct MfmaArgs {
+    const bf16_t* q;        // [n][H][D]
+    const bf16_t* k_pages;  // [page][G][slot][D]
+    const bf16_t* v_pages;  // [page][G][Dv][slot]
+    const int* positions;
+    const int* tok_entry;
+    const int* block_table;
+    const int* tiles;       // [n_tiles][2]: first row, rows (1..16), all of one request
+    const void* gate;       // gate[t * ldg + h], or null
+    bf16_t* out;            // [n][H][Dv]
+    long long ldg;
+    int n_tiles, H, G, page_size, max_blocks, num_pages, window, chunk, gate_f32;
+    float scale, cap;
+};
+
+__device__ __forceinline__ vt_lowp4_t load4(const bf16_t* p) { return *(const vt_lowp4_t*)p; }
+
+__global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
+    constexpr int D = VT_KEY_DIM, DV = VT_VALUE_DIM, NK = D / 16, NV = DV / 16;
+    const int lane = threadIdx.x & 63;
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= a.n_tiles * a.H) return;
+    const int tile = item / a.H, h = item % a.H;
+    const int kvh = h / (a.H / a.G);
+    const int first = a.tiles[2 * tile], rows = a.tiles[2 * tile + 1];
+    const int r = lane & 15, grp = lane >> 4;
+    const bool row_ok = r < rows;
+    const int t = first + (row_ok ? r : 0);
+    const int pos = a.positions[t];
+    const int pos_first = a.positions[first], pos_last = a.positions[first + rows - 1];
+    const int* bt = a.block_table + (size_t)a.tok_entry[first] * a.max_blocks;
+    const int ps = a.page_size;
+
+    int lo_r = a.chunk > 0 ? (pos / a.chunk) * a.chunk : 0;
+    if (a.window > 0) lo_r = max(lo_r, pos - a.window + 1);
+    int lo = a.chunk > 0 ? (pos_first / a.chunk) * a.chunk : 0;       // the first row's bound is the lowest
+    if (a.window > 0) lo = max(lo, pos_first - a.window + 1);
+
+    vt_lowp4_t qf[NK];
+    {
+        const bf16_t* qr = a.q + ((size_t)t * a.H + h) * D + grp * 4;
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) {
+            qf[kk] = load4(qr + kk * 16);
+            if (!row_ok) qf[kk] = (vt_lowp4_t){0, 0, 0, 0};
+        }
+    }
+    f32x4 acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const float nan = __int_as_float(0x7fc00000);
+
+    for (int kt = (lo / 16) * 16; kt <= pos_last; kt += 16) {
+        const int blk = kt / ps;
+        int pg = bt[blk];
+        const bool page_ok = pg >= 0 && pg < a.num_pages;
+        pg = page_ok ? pg : 0;
+        const int slot0 = kt - blk * ps;
+        const bf16_t* kp = a.k_pages + (((size_t)pg * a.G + kvh) * ps + slot0 + r) * D + grp * 4;
+        const bf16_t* vp = a.v_pages + (((size_t)pg * a.G + kvh) * DV + r) * ps + slot0 + grp * 4;
+        vt_lowp4_t kf[NK], vf[NV];
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) kf[kk] = load4(kp + kk * 16);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) vf[v] = load4(vp + (size_t)v * 16 * ps);
+        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) s = VT_MFMA_16X16X16(kf[kk], qf[kk], s);
+        float sc[4];
+        float mt = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int j = kt + grp * 4 + i;
+            float x = s[i] * a.scale;
+            if (a.cap > 0.f) {
+                // cap * tanh(x / cap), tanh(y) = 1 - 2 / (1 + e^(2y))
+                const float e = __expf(2.0f * x / a.cap);
+                x = a.cap * (1.0f - 2.0f / (1.0f + e));
+            }
+            const bool seen = row_ok && j <= pos && j >= lo_r;
+            x = seen ? (page_ok ? x : nan) : -INFINITY;      // a missing page must show, not pass as a masked key
+            sc[i] = x;
+            mt = fmaxf(mt, x);
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m, mt);
+        const float mref = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
+        float p[4], psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            p[i] = __expf(sc[i] - mref);
+            psum += p[i];
+        }
+        l = l * alpha + psum;
+        m = m_new;
+        const unsigned p01 = vt_pack2(p[0], p[1]), p23 = vt_pack2(p[2], p[3]);
+        struct { unsigned a, b; } pk = {p01, p23};
+        const vt_lowp4_t pf = __builtin_bit_cast(vt_lowp4_t, pk);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            acc[v] *= alpha;
+            acc[v] = VT_MFMA_16X16X16(vf[v], pf, acc[v]);
+        }
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!row_ok) return;
+    float gate = 1.f;
+    if (a.gate) {
+        const size_t gi = (size_t)t * a.ldg + h;
+        const float z = a.gate_f32 ? ((const float*)a.gate)[gi] : bf16_to_f32(((const bf16_t*)a.gate)[gi]);
+        gate = 1.0f / (1.0f + expf(-z));
+    }
+    const float f = gate / l;
+    bf16_t* o = a.out + ((size_t)t * a.H + h) * DV + grp * 4;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        struct { unsigned a, b; } ok = {vt_pack2(acc[v][0] * f, acc[v][1] * f), vt_pack2(acc[v][2] * f, acc[v][3] * f)};
+        *(uint2*)(o + v * 16) = __builtin_bit_cast(uint2, ok);
+    }
+}
+
+extern "C" int vt_attn_masked_mfma_dims(int* key_dim, int* value_dim) {
+    *key_dim = VT_KEY_DIM;
+    *value_dim = VT_VALUE_DIM;
+    return 0;
+}
+
+extern "C" int vt_attn_masked_mfma(const void* q, const void* k_pages, const void* v_pages, const int* positions,
+                                   const int* tok_entry, const int* block_table, const int* tiles, int n_tiles,
+                                   const void* gate, int gate_dtype, long long ldg, void* out, int H, int G, int D, int Dv,
+                                   int page_size, int max_blocks, int num_pages, int window, int chunk, float scale,
+                                   float cap, hipStream_t stream) {
+    VT_REQUIRE(D == VT_KEY_DIM && Dv == VT_VALUE_DIM, "vt_attn_masked_mfma: built for heads of %d/%d, called with %d/%d",
+               VT_KEY_DIM, VT_VALUE_DIM, D, Dv);
+    VT_REQUIRE(n_tiles >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked_mfma: bad heads %d/%d", H, G);
+    VT_REQUIRE(page_size > 0 && page_size % 16 == 0 && max_blocks > 0 && num_pages > 0,
+               "vt_attn_masked_mfma: pages of %d keys (a multiple of 16)", page_size);
+    VT_REQUIRE(window >= 0 && chunk >= 0 && cap >= 0.f, "vt_attn_masked_mfma: bad mask or cap");
+    VT_REQUIRE(!gate || gate_dtype == VT_F32 || gate_dtype == VT_BF16, "vt_attn_masked_mfma: gate dtype %d", gate_dtype);
+    if (n_tiles == 0) return 0;
+    MfmaArgs a;
+    a.q = (const bf16_t*)q; a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages; a.positions = positions;
+    a.tok_entry = tok_entry; a.block_table = block_table; a.tiles = tiles; a.gate = gate; a.out = (bf16_t*)out; a.ldg = ldg;
+    a.n_tiles = n_tiles; a.H = H; a.G = G; a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages;
+    a.window = window; a.chunk = chunk; a.gate_f32 = gate_dtype == VT_F32; a.scale = scale; a.cap = cap;
+    const long long items = (long long)n_tiles * H;
+    attn_masked_mfma_kernel<<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(a);
+    VT_CHECK_LAUNCH("vt_attn_masked_mfma");
+    return 0;
+}

@@ -9,10 +9,11 @@
 //   vt_short_conv:        y[t][c] = silu(sum_j taps[c][j] x[t - (K-1) + j][c]); inputs before a request's first token
 //                         of this step come from its state (zeros at the start of a sequence).
 //   vt_short_conv_carry:  the last K-1 inputs of every request go into its state (after vt_short_conv has read it).
-//   vt_delta_rule:        the recurrence.  A block takes 64 value columns of one (request, head); four lanes share a
-//                         column, each holding a quarter of its D state elements in registers.  Tokens are taken in
-//                         tiles of 16 through LDS; every token is computed by the same instructions in the same
-//                         order whatever the tile, so a result does not depend on how the request was cut into steps.
+//   vt_delta_rule:        the recurrence.  A block takes 16 value columns of one (request, head); the 16 lanes of a
+//                         row share a column, each holding a sixteenth of its D state elements in registers, and
+//                         add their shares up by rotations within the row.  Tokens are taken in tiles of 16 through
+//                         LDS; every token is computed by the same instructions in the same order whatever the
+//                         tile, so a result does not depend on how the request was cut into steps.
 //   vt_gated_rmsnorm:     out = o / rms(o) * w * silu(gate), per (token, head).
 #include "vt_common.h"
 #include <math.h>
@@ -130,7 +131,7 @@ struct DeltaArgs {
     const float* ba;        // [n][2H]: beta logits, then decay logits
     const float* a_log;     // [H]
     const float* dt_bias;   // [H]
-    float* state;           // slot s: state + s * slot_stride, [H][D][Dv]
+    float* state;           // slot s: state + s * slot_stride, [H][Dv][D]
     const int* entry_start;
     const int* slots;
     float* o;               // [n][H][Dv]
@@ -139,12 +140,22 @@ struct DeltaArgs {
 };
 
 #define DELTA_TILE 16
-#define DELTA_COLS 64
+#define DELTA_COLS 16
 
-// DS: state elements per lane (a quarter of D, rounded up to a power of two from 8 to 64)
+// the sum of v over the 16 lanes of a row (lanes 16 r .. 16 r + 15), in every one of them: four rotations within the row
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
+    v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
+    return v;
+}
+
+// DS: state elements per lane (a sixteenth of D, rounded up to a power of two).  Lane r of a column's 16 holds the
+// elements d = 16 i + r, i < DS: a row of lanes reads 16 consecutive floats of LDS or of the state at a time.
 template <typename TI, int DS>
 __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
-    constexpr int DP = 4 * DS;                        // D padded
+    constexpr int DP = 16 * DS;                       // D padded
     __shared__ float qs[DELTA_TILE][DP];
     __shared__ float ks[DELTA_TILE][DP];
     __shared__ float vs[DELTA_TILE][DELTA_COLS];
@@ -152,13 +163,14 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
 
     const int e = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * DELTA_COLS;
     const int tid = threadIdx.x;
-    const int r = tid & 3, col = col0 + (tid >> 2);
+    const int r = tid & 15, cl = tid >> 4, col = col0 + cl;
     const bool col_ok = col < a.Dv;
     const int D = a.D, Dv = a.Dv, H = a.H, G = a.G;
     const int kh = h / (H / G);
     const int C = 2 * G * D + H * Dv;
     const int start = a.entry_start[e], end = a.entry_start[e + 1];
-    float* S_mem = a.state + (size_t)a.slots[e] * a.slot_stride + (size_t)h * D * Dv;
+    // the state of a head is kept [Dv][D]: a column's D elements lie together
+    float* S_mem = a.state + (size_t)a.slots[e] * a.slot_stride + ((size_t)h * Dv + (col_ok ? col : 0)) * D;
     const TI* x = (const TI*)a.qkv;
     const float decay_rate = expf(a.a_log[h]);
     const float bias = a.dt_bias[h];
@@ -167,8 +179,8 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
     float S[DS];
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = r * DS + i;
-        S[i] = (col_ok && d < D) ? S_mem[(size_t)d * Dv + col] : 0.f;
+        const int d = 16 * i + r;
+        S[i] = (col_ok && d < D) ? S_mem[d] : 0.f;
     }
 
     for (int t0 = start; t0 < end; t0 += DELTA_TILE) {
@@ -185,8 +197,8 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
             qs[tt][d] = qv;
             ks[tt][d] = kv;
         }
-        for (int i = tid; i < DELTA_TILE * DELTA_COLS; i += 256) {
-            const int tt = i / DELTA_COLS, j = i % DELTA_COLS;
+        {
+            const int tt = tid / DELTA_COLS, j = tid % DELTA_COLS;      // 16 tokens x 16 columns = the block's threads
             vs[tt][j] = (tt < nt && col0 + j < Dv)
                             ? load_f32<TI>(x, (size_t)(t0 + tt) * C + (size_t)2 * G * D + (size_t)h * Dv + col0 + j) : 0.f;
         }
@@ -206,33 +218,36 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
         }
         __syncthreads();
         for (int tt = 0; tt < nt; ++tt) {
+            // with k' = rk k and q' = rq q:  S <- g S;  u = beta (v - k'.S);  S <- S + k' u;  o = q'.S
             const float g = g_s[tt], beta = beta_s[tt], rq = rq_s[tt], rk = rk_s[tt];
-            const float* kk = &ks[tt][r * DS];
-            const float* qq = &qs[tt][r * DS];
+            float kk[DS], qq[DS];
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                kk[i] = ks[tt][16 * i + r];
+                qq[i] = qs[tt][16 * i + r];
+            }
             float dot = 0.f;
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
                 S[i] *= g;
-                dot = fmaf(kk[i] * rk, S[i], dot);
+                dot = fmaf(kk[i], S[i], dot);
             }
-            dot += __shfl_xor(dot, 1, 64);
-            dot += __shfl_xor(dot, 2, 64);
-            const float u = beta * (vs[tt][tid >> 2] - dot);
+            dot = row16_sum(dot);
+            const float u = beta * (vs[tt][cl] - rk * dot) * rk;
             float out = 0.f;
 #pragma unroll
             for (int i = 0; i < DS; ++i) {
-                S[i] = fmaf(kk[i] * rk, u, S[i]);
-                out = fmaf(qq[i] * rq, S[i], out);
+                S[i] = fmaf(kk[i], u, S[i]);
+                out = fmaf(qq[i], S[i], out);
             }
-            out += __shfl_xor(out, 1, 64);
-            out += __shfl_xor(out, 2, 64);
-            if (r == 0 && col_ok) a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = out;
+            out = row16_sum(out);
+            if (r == 0 && col_ok) a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = rq * out;
         }
     }
 #pragma unroll
     for (int i = 0; i < DS; ++i) {
-        const int d = r * DS + i;
-        if (col_ok && d < D) S_mem[(size_t)d * Dv + col] = S[i];
+        const int d = 16 * i + r;
+        if (col_ok && d < D) S_mem[d] = S[i];
     }
 }
 
@@ -248,13 +263,14 @@ extern "C" int vt_delta_rule(const void* qkv, int dtype, const float* ba, const 
     a.qkv = qkv; a.ba = ba; a.a_log = a_log; a.dt_bias = dt_bias; a.state = state; a.entry_start = entry_start;
     a.slots = slots; a.o = o; a.slot_stride = slot_stride; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
     const dim3 grid(n_entries, H, (Dv + DELTA_COLS - 1) / DELTA_COLS);
-    const int quarter = (D + 3) / 4;
+    const int share = (D + 15) / 16;
 #define VT_DELTA(TI)                                                                          \
     do {                                                                                      \
-        if (quarter <= 8) delta_rule_kernel<TI, 8><<<grid, 256, 0, stream>>>(a);              \
-        else if (quarter <= 16) delta_rule_kernel<TI, 16><<<grid, 256, 0, stream>>>(a);       \
-        else if (quarter <= 32) delta_rule_kernel<TI, 32><<<grid, 256, 0, stream>>>(a);       \
-        else delta_rule_kernel<TI, 64><<<grid, 256, 0, stream>>>(a);                          \
+        if (share <= 1) delta_rule_kernel<TI, 1><<<grid, 256, 0, stream>>>(a);                \
+        else if (share <= 2) delta_rule_kernel<TI, 2><<<grid, 256, 0, stream>>>(a);           \
+        else if (share <= 4) delta_rule_kernel<TI, 4><<<grid, 256, 0, stream>>>(a);           \
+        else if (share <= 8) delta_rule_kernel<TI, 8><<<grid, 256, 0, stream>>>(a);           \
+        else delta_rule_kernel<TI, 16><<<grid, 256, 0, stream>>>(a);                          \
     } while (0)
     if (dtype == VT_F32) VT_DELTA(float);
     else if (dtype == VT_BF16) VT_DELTA(bf16_t);

@@ -34,7 +34,9 @@ BASE_LIBS = ["vt_elementwise", "vt_gemm_f32", "vt_gemm_bf16", "vt_attn_f32", "vt
 DEFAULT_HEAD_DIMS = list(range(16, 257, 16))
 # The libraries that handle 16-bit values are built once for bfloat16 and once for float16 (-DVT_LOWP_F16: the same
 # sources with the other conversion and the other matrix instruction); the float16 build's name ends in _f16.
-HALF_LIBS = ("vt_elementwise", "vt_gemm_bf16", "vt_attn_bf16", "vt_attn_masked", "vt_delta")
+HALF_LIBS = ("vt_elementwise", "vt_gemm_bf16", "vt_attn_bf16", "vt_attn_masked", "vt_attn_masked_mfma", "vt_delta")
+# the matrix-core kernel of the masked attention is built per (key size, value size) of a head
+DEFAULT_MASKED_DIMS = [(64, 64), (128, 128), (64, 80), (32, 48), (16, 16)]
 
 
 class KernelBuildError(RuntimeError):
@@ -92,6 +94,12 @@ def lib_spec(name: str, head_dim: Optional[int] = None, half: bool = False) -> T
             raise ValueError("vt_attn_bf16 is built per head size")
         defines["VT_HEAD_DIM"] = str(head_dim)
         return f"vt_attn_bf16_d{head_dim}{suffix}", os.path.join(CSRC, "vt_attn_bf16.hip"), defines
+    if name == "vt_attn_masked_mfma":
+        if not isinstance(head_dim, (tuple, list)) or len(head_dim) != 2:
+            raise ValueError("vt_attn_masked_mfma is built per (key size, value size)")
+        defines["VT_KEY_DIM"], defines["VT_VALUE_DIM"] = str(int(head_dim[0])), str(int(head_dim[1]))
+        return (f"vt_attn_masked_mfma_k{int(head_dim[0])}_v{int(head_dim[1])}{suffix}",
+                os.path.join(CSRC, "vt_attn_masked_mfma.hip"), defines)
     return name + suffix, os.path.join(CSRC, name + ".hip"), defines
 
 
@@ -157,6 +165,7 @@ def build_all(head_dims: Iterable[int] = DEFAULT_HEAD_DIMS, force: bool = True, 
     head_dims = list(head_dims)
     tasks = [(n, None, False) for n in BASE_LIBS] + [("vt_attn_bf16", d, False) for d in head_dims]
     tasks += [(n, None, True) for n in BASE_LIBS if n in HALF_LIBS] + [("vt_attn_bf16", d, True) for d in head_dims]
+    tasks += [("vt_attn_masked_mfma", kv, half) for kv in DEFAULT_MASKED_DIMS for half in (False, True)]
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, 16))) as ex:
         return list(ex.map(lambda t: compile_lib(t[0], t[1], force=force, verbose=verbose, half=t[2]), tasks))
 

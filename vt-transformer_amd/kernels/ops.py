@@ -668,7 +668,7 @@ def qk_prepare(x: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch
     """x [n, >= (H + G) D + G Dv]: query heads, key heads, value heads.  Rotates the leading 2 * cos.shape[1] elements
     of every query and key head by the tables' angles at `positions`, divides each head by its root mean square
     (eps inside the root) unless unit_rms_eps is None, writes queries to q_out [n, H * D] and, with write_kv, keys and
-    values into their pages ([page][kv][slot][D] and [page][kv][slot][Dv])."""
+    values into their pages ([page][kv][slot][D] and, transposed, [page][kv][Dv][slot])."""
     n = x.shape[0]
     _chk(x, "qk_prepare.x")
     need = (n_heads + (n_kv if write_kv else 0)) * key_dim + (n_kv * value_dim if write_kv else 0)
@@ -695,7 +695,7 @@ def qk_prepare(x: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch
         num_pages, kvh, page_size, d = k_pages.shape
         if (kvh, d) != (n_kv, key_dim):
             raise KernelError(f"qk_prepare.k_pages: shape {tuple(k_pages.shape)} does not fit kv heads {n_kv} x {key_dim}")
-        _chk(v_pages, "qk_prepare.v_pages", q_out.dtype, (num_pages, n_kv, page_size, value_dim))
+        _chk(v_pages, "qk_prepare.v_pages", q_out.dtype, (num_pages, n_kv, value_dim, page_size))
         _chk(block_table, "qk_prepare.block_table", torch.int32)
         max_blocks = block_table.shape[1]
     _run(load_lib("vt_attn_masked", half=_half(x, q_out)), "vt_qk_prepare", _ptr(x), _i(_code(x)),
@@ -717,7 +717,7 @@ def attention_masked(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
     dt = q.dtype
     _chk(q, "attention_masked.q", None, (n, n_heads * key_dim))
     _chk(k_pages, "attention_masked.k_pages", dt, (num_pages, n_kv, page_size, key_dim))
-    _chk(v_pages, "attention_masked.v_pages", dt, (num_pages, n_kv, page_size, value_dim))
+    _chk(v_pages, "attention_masked.v_pages", dt, (num_pages, n_kv, value_dim, page_size))
     _chk(out, "attention_masked.out", dt, (n, n_heads * value_dim))
     _chk(positions, "attention_masked.positions", torch.int32, (n,))
     _chk(tok_entry, "attention_masked.tok_entry", torch.int32, (n,))
@@ -737,6 +737,49 @@ def attention_masked(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
          _ptr(positions), _ptr(tok_entry), _ptr(block_table), gptr, _i(gcode), ctypes.c_longlong(ldg), _ptr(out), _i(n),
          _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size), _i(block_table.shape[1]), _i(num_pages),
          _i(window), _i(chunk), _f(scale), _f(cap), _stream())
+    return out
+
+
+def attention_masked_mfma_takes(key_dim: int, value_dim: int, page_size: int) -> bool:
+    """Whether the matrix-core kernel takes heads and pages of these sizes."""
+    return (key_dim % 16 == 0 and value_dim % 16 == 0 and 16 <= key_dim <= 256 and 16 <= value_dim <= 256
+            and page_size % 16 == 0)
+
+
+def attention_masked_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, positions: torch.Tensor,
+                          tok_entry: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor, out: torch.Tensor,
+                          n_heads: int, n_kv: int, key_dim: int, value_dim: int, scale: float, cap: float = 0.0,
+                          window: int = 0, chunk: int = 0, gate: Optional[torch.Tensor] = None,
+                          gate_column: int = 0) -> torch.Tensor:
+    """attention_masked for the 16-bit types on the matrix cores.  tiles: int32 [n_tiles, 2], (first row, rows) of
+    runs of up to 16 consecutive tokens of one request that together cover every token of the step once."""
+    n = q.shape[0]
+    num_pages, kvh, page_size, d = k_pages.shape
+    dt = _lowp(q, "attention_masked_mfma.q")
+    if not attention_masked_mfma_takes(key_dim, value_dim, page_size):
+        raise KernelError(f"attention_masked_mfma: heads of {key_dim}/{value_dim} and pages of {page_size} "
+                          f"(multiples of 16 up to 256)")
+    _chk(q, "attention_masked_mfma.q", dt, (n, n_heads * key_dim))
+    _chk(k_pages, "attention_masked_mfma.k_pages", dt, (num_pages, n_kv, page_size, key_dim))
+    _chk(v_pages, "attention_masked_mfma.v_pages", dt, (num_pages, n_kv, value_dim, page_size))
+    _chk(out, "attention_masked_mfma.out", dt, (n, n_heads * value_dim))
+    _chk(positions, "attention_masked_mfma.positions", torch.int32, (n,))
+    _chk(tok_entry, "attention_masked_mfma.tok_entry", torch.int32, (n,))
+    _chk(block_table, "attention_masked_mfma.block_table", torch.int32)
+    _chk(tiles, "attention_masked_mfma.tiles", torch.int32)
+    if tiles.numel() % 2:
+        raise KernelError("attention_masked_mfma.tiles: pairs of (first row, rows)")
+    gptr, gcode, ldg = ctypes.c_void_p(0), F32, 0
+    if gate is not None:
+        _chk(gate, "attention_masked_mfma.gate")
+        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads:
+            raise KernelError(f"attention_masked_mfma.gate: shape {tuple(gate.shape)} has no {n_heads} columns from {gate_column}")
+        gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
+        gcode, ldg = _code(gate), gate.stride(0)
+    _run(load_lib("vt_attn_masked_mfma", (key_dim, value_dim), half=_half(q, gate)), "vt_attn_masked_mfma", _ptr(q), _ptr(k_pages),
+         _ptr(v_pages), _ptr(positions), _ptr(tok_entry), _ptr(block_table), _ptr(tiles), _i(tiles.numel() // 2), gptr,
+         _i(gcode), ctypes.c_longlong(ldg), _ptr(out), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size),
+         _i(block_table.shape[1]), _i(num_pages), _i(window), _i(chunk), _f(scale), _f(cap), _stream())
     return out
 
 
@@ -796,7 +839,7 @@ def short_conv_carry(x: torch.Tensor, channels: int, k: int, state: torch.Tensor
 def delta_rule(qkv: torch.Tensor, ba: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor,
                entry_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, key_dim: int,
                value_dim: int) -> torch.Tensor:
-    """The gated delta rule over the tokens of every entry, from and into state[slot] ([H, D, Dv] float32).
+    """The gated delta rule over the tokens of every entry, from and into state[slot] ([H, Dv, D] float32).
     qkv [n, 2 G D + H Dv]: queries, keys (G heads of D), values (H heads of Dv); ba [n, 2 H] float32: logits of the
     write strength and of the decay.  out [n, H * Dv] float32."""
     n = qkv.shape[0]

@@ -67,7 +67,7 @@ class GatedDeltaMixer(Part):
 
     def state_need(self) -> Optional[StateNeed]:
         """One float32 row per request: the convolutions' last taps - 1 inputs [taps - 1][channels], then the heads'
-        matrices [H][D][Dv]."""
+        matrices [H][Dv][D]."""
         return StateNeed((self.conv_floats + self.rule_floats,), torch.float32)
 
     def tensors(self) -> Dict[str, TensorDecl]:

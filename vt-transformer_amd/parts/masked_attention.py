@@ -22,6 +22,7 @@ from __future__ import annotations
 import math
 from typing import Callable, Dict, Optional
 
+import numpy as np
 import torch
 
 from ..config.base import PartSpec
@@ -81,11 +82,33 @@ class MaskedAttention(Part):
         return (self.nh + self.nkv) * self.d + self.nkv * self.dv
 
     def cache_need(self) -> Optional[CacheNeed]:
-        """Keys [kv head][slot][D] and values [kv head][slot][Dv] in the runtime's dtype.  The mask's reach bounds how
-        long a key lives: with chunks, a key is never seen from `chunk` or more positions later."""
+        """Keys [kv head][slot][D] and values transposed, [kv head][Dv][slot] (the matrix-core kernel reads four keys of
+        one value element with one load), in the runtime's dtype.  The mask's reach bounds how long a key lives: with
+        chunks, a key is never seen from `chunk` or more positions later."""
         reach = [w for w in (self.window, self.chunk) if w > 0]
-        return CacheNeed((PageTensor("k", (self.nkv, self.d), slot_axis=1), PageTensor("v", (self.nkv, self.dv), slot_axis=1)),
-                         window=min(reach) if reach else 0, page_multiple=1)
+        return CacheNeed((PageTensor("k", (self.nkv, self.d), slot_axis=1), PageTensor("v", (self.nkv, self.dv), slot_axis=2)),
+                         window=min(reach) if reach else 0, page_multiple=16 if self._matrix_cores() else 1)
+
+    def _matrix_cores(self) -> bool:
+        """Whether portions of prompts go to the matrix-core kernel: a 16-bit runtime and heads in multiples of 16."""
+        return self.rt.lowp and ops.attention_masked_mfma_takes(self.d, self.dv, 16)
+
+    TILE_ROWS = 16
+
+    def prepare_step(self, ctx) -> Optional[Dict[tuple, np.ndarray]]:
+        """The matrix-core kernel's work for a step that brings more than single tokens: runs of up to 16 consecutive
+        tokens of one request, (first row, rows).  One list serves every layer of this kind."""
+        if not self._matrix_cores() or ctx.single_token:
+            return None
+        key = ("masked_attention.tiles", self.TILE_ROWS)
+        if key in ctx.extra_host:
+            return None
+        start = np.asarray(ctx.h_entry_start, dtype=np.int64)
+        tiles = []
+        for e in range(len(start) - 1):
+            for first in range(int(start[e]), int(start[e + 1]), self.TILE_ROWS):
+                tiles.append((first, min(self.TILE_ROWS, int(start[e + 1]) - first)))
+        return {key: np.asarray(tiles, dtype=np.int32).reshape(-1)}
 
     def state_need(self) -> Optional[StateNeed]:
         return None
@@ -132,6 +155,12 @@ class MaskedAttention(Part):
         ops.qk_prepare(y, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, nkv,
                        d, dv, self.unit_rms_eps)
         out = rt.buffer("mattn.out", (n, nh * dv), rt.dtype)
+        tiles = ctx.extra.get(("masked_attention.tiles", self.TILE_ROWS)) if self._matrix_cores() and not ctx.single_token else None
+        if tiles is not None and cache["k"].shape[2] % 16 == 0:
+            ops.attention_masked_mfma(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, tiles, out,
+                                      nh, nkv, d, dv, self.scale, self.softcap, self.window, self.chunk,
+                                      gate=y if self.head_gate else None, gate_column=self._gate_column)
+            return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o)
         ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
                              dv, self.scale, self.softcap, self.window, self.chunk,
                              gate=y if self.head_gate else None, gate_column=self._gate_column)
