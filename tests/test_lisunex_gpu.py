@@ -231,7 +231,7 @@ def test_gated_delta_part(dtype, nh, kvh, d, dv, taps):
         w = {k: v for k, v in w.items() if "conv" not in k}
     mixer.load(w.__getitem__, rt)
     runner = ModelRunner(OneMixer(mixer), rt, 16, 256, 3, 256)
-    assert runner.storage.state[0].shape == (3, (taps - 1) * (2 * kvh * d + nh * dv) + nh * d * dv)
+    assert runner.storage.state[0].shape == (3 + 1, (taps - 1) * (2 * kvh * d + nh * dv) + nh * d * dv)
     x = (torch.randn(t, width, generator=torch.Generator().manual_seed(8)) * 0.8).to(dtype)
     wd = {k[2:].replace("_proj.weight", "").replace("_conv.weight", ".conv").replace("norm.weight", "norm"): v.double()
           for k, v in w.items()}
@@ -342,3 +342,33 @@ def test_trace_run_with_a_lisunex_folder(folders, tmp_path):
     got = rh.run_trace_run(folder, "float32", steps, str(tmp_path / "out"), rh.max_live_tokens(steps), vocab,
                            extra_args=("--max-requests", "2"))
     check_logits(folder, reqs, steps, got, "float32")
+
+
+def test_captured_decoding_steps_move_the_state_once(folders):
+    """Decoding through captured steps (bfloat16): the launch-by-launch run in front of a capture is the step itself,
+    later steps are replays, padding entries use the state row that nobody owns; the logits are those of the same
+    schedule launched step by step, bit for bit, and the plain implementation's within rounding."""
+    folder, vocab = folders["A"], CONFIGS["A"]["vocab"]
+    reqs = rh.random_requests(vocab, [30, 12, 21], seed=31)
+    steps, nxt = [], {r: 6 for r in reqs}
+    steps.append({"step": 0, "entries": [{"id": r, "tokens": t[:6], "want": [5]} for r, t in reqs.items()], "end": []})
+    while nxt:
+        live = list(nxt)
+        entries = [{"id": r, "tokens": reqs[r][nxt[r]:nxt[r] + 1], "want": [0]} for r in live]
+        end = []
+        for r in live:
+            nxt[r] += 1
+            if nxt[r] == len(reqs[r]):
+                end.append(r)
+                del nxt[r]
+        steps.append({"step": len(steps), "entries": entries, "end": end})
+    plain = make_runner(folder, "bfloat16", pool_tokens=192, max_requests=3)
+    got_plain = rh.run_in_process(plain, steps)
+    graphs = make_runner(folder, "bfloat16", pool_tokens=192, max_requests=3)
+    graphs.decode_graphs = True
+    assert graphs.replays(3) and not graphs._stateless
+    got = rh.run_in_process(graphs, steps)
+    assert graphs._graphs, "no decoding step was captured"
+    for k in got_plain:
+        assert np.array_equal(got[k], got_plain[k]), f"step {k} differs between replayed and launched steps"
+    check_logits(folder, reqs, steps, got, "bfloat16")

@@ -467,7 +467,7 @@ def test_toy_mixer_with_state_toy_position_encoding_and_toy_routing():
     model.load(w.__getitem__)
     runner = make_runner(model, pool_tokens=128, page_size=16, max_requests=2, max_seq_len=128)
     assert [s is not None for s in runner.storage.state] == [True, False, True, False]    # state slots for the toy
-    assert runner.storage.state[0].shape == (2, 48)
+    assert runner.storage.state[0].shape == (2 + 1, 48)        # (one row more than slots: the padding entries')
     assert runner.storage.n_groups == 1 and runner.storage.pages[0]["k"].shape[0] == 2               # pages for attention only
     wd = {n: t.double() for n, t in w.items()}
     rs = np.random.RandomState(1)

@@ -128,11 +128,13 @@ class CacheStorage:
             self.pages.append({t.name: torch.zeros((members[g], pages[g]) + t.page_shape(self.page_size),
                                                    dtype=t.dtype or rt.dtype, device=rt.device) for t in need.tensors})
         self.writes = [e.cache_from is None for e in schedule]
-        # fixed-size state per request and schedule entry (none for attention)
+        # fixed-size state per request and schedule entry (none for attention): one row per state slot, and one more
+        # (`spare_slot`) that belongs to nobody, for the padding entries of a captured decoding step
+        self.spare_slot = int(max_requests)
         self.state: List[Optional[torch.Tensor]] = []
         for need in state_needs:
             self.state.append(None if need is None else
-                              torch.zeros((max_requests,) + tuple(need.shape), dtype=need.dtype, device=rt.device))
+                              torch.zeros((max_requests + 1,) + tuple(need.shape), dtype=need.dtype, device=rt.device))
 
     @property
     def num_pages(self) -> int:

@@ -112,17 +112,17 @@ class ModelRunner:
         self.steps = 0
         self.tokens = 0
         self._staging = HostStaging(torch.int32)
-        # Decoding steps of a 16-bit model are captured once per batch size and replayed, unless a mixer keeps
-        # state of its own between steps (the warm-up run before a capture would advance it twice) or a part does
-        # not declare that its step can be replayed.  This is decided here, once, for the whole model: one part that
-        # is stateful or says nothing keeps every step of the model on the launch-by-launch path (and the engine,
-        # which asks `replays()`, then never starts a step ahead of the host); the other parts lose nothing but that.
+        # Decoding steps of a 16-bit model are captured once per batch size and replayed, unless a part does not
+        # declare that its step can be replayed.  This is decided here, once, for the whole model: one part that
+        # says nothing keeps every step of the model on the launch-by-launch path (and the engine, which asks
+        # `replays()`, then never starts a step ahead of the host); the other parts lose nothing but that.  A model
+        # whose mixers keep state of their own between steps is replayed too: the launch-by-launch run in front of
+        # a capture is then the step itself (`_step_decode_graph`), so the state moves once.
         self.decode_graphs = False
         self._graphs: Dict[int, _DecodeGraph] = {}
         self._stateless = all(s is None for s in self.storage.state)
         parts = model.parts() if hasattr(model, "parts") else None
-        self._replayable = (self._stateless and parts is not None
-                            and all(bool(getattr(p, "replayable", False)) for p in parts))
+        self._replayable = parts is not None and all(bool(getattr(p, "replayable", False)) for p in parts)
         # parts that plan work of their own for a step (PagedAttention does)
         known = parts if parts is not None else [getattr(layer, "mixer", None) for layer in model.layers]
         self._preparers = [p for p in known if p is not None and hasattr(p, "prepare_step")]
@@ -154,7 +154,8 @@ class ModelRunner:
             lens = np.concatenate([lens, np.ones(n_pad, np.int64)])
             pos0 = np.concatenate([pos0, np.zeros(n_pad, np.int64)])
             ids = np.concatenate([ids, np.zeros(n_pad, np.int64)])
-            slots = np.concatenate([slots, np.zeros(n_pad, np.int64)])
+            # (a padding entry's state, if the model keeps any, is the row that no request owns)
+            slots = np.concatenate([slots, np.full(n_pad, self.storage.spare_slot, np.int64)])
         n_all = n_entries + n_pad
         start = np.zeros(n_all + 1, dtype=np.int64)
         np.cumsum(lens, out=start[1:])
@@ -299,15 +300,18 @@ class ModelRunner:
         fixed_blocks = -(-self.max_seq_len // self.cache.page_size)
         h = self._host_arrays(entries, pad_to=b, fixed_blocks=fixed_blocks)
         all_rows = np.arange(b, dtype=np.int32)     # logits of every entry; the wanted ones are picked afterwards
+        ran = False
         with self.rt.scoped(f"graph{b}:"):
             if g is None:
                 g = _DecodeGraph()
                 g.ctx = StepContext(self.rt, self.max_seq_len)
                 g.meta = self._fill_context(g.ctx, h, all_rows, None)
+                self._feed_ids(g, ids_dev, n)
                 caches = self.storage.layer_caches(g.ctx.block_tables)
                 # once eagerly: loads the libraries and makes every scratch buffer, so the capture allocates nothing
                 self.model.forward(g.ctx, caches, self.storage.state)
                 torch.cuda.synchronize()
+                ran = not self._stateless   # a model with state of its own has now made this step: no replay on top
                 g.graph = torch.cuda.CUDAGraph()
                 # No cyclic garbage collection while the step is recorded: it may destroy an object that owns device
                 # or pinned memory, events or another recorded graph (an engine that the caller has dropped), and
@@ -323,8 +327,9 @@ class ModelRunner:
                 self._graphs[b] = g
             else:
                 self._fill_context(g.ctx, h, all_rows, g.meta)
-            self._feed_ids(g, ids_dev, n)
-            g.graph.replay()
+            if not ran:
+                self._feed_ids(g, ids_dev, n)
+                g.graph.replay()
         # what the next step can patch instead of building anew: the host copy of the metadata and where its parts lie
         g.rps, g.h, g.flat = rps, h, self._last_flat
         g.table_lens = [[len(self.cache.get(e.rid).tables[gi]) for e in entries] for gi in range(self.storage.n_groups)]

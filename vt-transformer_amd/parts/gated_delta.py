@@ -31,7 +31,8 @@ from .linear import linear, linear_f32_out
 
 @MIXERS.register("gated_delta")
 class GatedDeltaMixer(Part):
-    replayable = False      # it keeps state of its own between steps
+    replayable = True       # a decoding step's launches depend on the number of entries only; its state lies in device
+                            # memory and is found by the slots of the step's metadata
 
     def __init__(self, *, rt: Runtime, width: int, prefix: str, num_heads: int, num_kv_heads: int, key_dim: int,
                  value_dim: int, conv_taps: int, norm_eps: float, shared: Optional[dict] = None,

@@ -33,7 +33,7 @@ from .linear import linear
 
 @MIXERS.register("masked_attention")
 class MaskedAttention(Part):
-    replayable = False      # (its launches' grids follow the step's tokens only, but nobody has replayed it yet)
+    replayable = True       # a decoding step's launches depend on the number of entries only
 
     def __init__(self, *, rt: Runtime, width: int, prefix: str, num_heads: int, num_kv_heads: int, key_dim: int,
                  value_dim: Optional[int] = None, qkv_bias: bool = False, position: Optional[PartSpec] = None,
