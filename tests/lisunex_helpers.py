@@ -13,8 +13,10 @@ import torch
 import plain_lisunex as pl
 
 # root mean square of a row's error (its mean taken off) over the root mean square of the row's logits (theirs too):
-# bfloat16 rounds every activation to eight bits, about 4e-3 each, through up to seven layer runs of these weights
-TOL = {"float32": 3e-5, "bfloat16": 3e-2}
+# bfloat16 rounds every activation to eight bits, about 4e-3 each, through up to seven layer runs of these weights; a
+# portion of more than 64 tokens also gets its projections' results in 16 bits (the GEMM library's), the logits of the
+# delta rule's decay among them, which these weights make steep
+TOL = {"float32": 3e-5, "bfloat16": 4e-2}
 
 
 def attention_layer(heads=4, kv_heads=2, dim=32, vdim=48, scale=0.2, softcap=15.0, chunk=24, rot_dims=8, base=10000.0,

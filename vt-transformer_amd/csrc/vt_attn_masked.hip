@@ -55,7 +55,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(PrepArgs a) {
         page_row = (size_t)page_no * a.G * a.page_size + page_slot;
     }
     const int units = a.H + (a.write_kv ? 2 * a.G : 0);
-    for (int u = wave; u < units; u += nw) {
+    for (int u = blockIdx.y * nw + wave; u < units; u += nw * gridDim.y) {
         if (u < a.H + a.G) {
             // a query or key head: rotate, then scale to unit root mean square
             const bool is_q = u < a.H;
@@ -128,9 +128,12 @@ extern "C" int vt_qk_prepare(const void* x, int x_dtype, long long ldx, const fl
     a.q_out = q_out; a.k_pages = k_pages; a.v_pages = v_pages; a.ldx = ldx; a.H = H; a.G = G; a.D = D; a.Dv = Dv; a.rot = rot;
     a.max_pos = max_pos; a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages; a.write_kv = write_kv;
     a.unit_rms = unit_rms; a.eps = eps;
-    if (x_dtype == VT_F32 && cache_dtype == VT_F32) qk_prepare_kernel<float, float><<<n, 256, 0, stream>>>(a);
-    else if (x_dtype == VT_F32 && cache_dtype == VT_BF16) qk_prepare_kernel<float, bf16_t><<<n, 256, 0, stream>>>(a);
-    else if (x_dtype == VT_BF16 && cache_dtype == VT_BF16) qk_prepare_kernel<bf16_t, bf16_t><<<n, 256, 0, stream>>>(a);
+    // few tokens: a wave per head, over several blocks per token; many tokens: a block per token goes through its heads
+    const int units = H + (write_kv ? 2 * G : 0);
+    const dim3 grid(n, n >= 1024 ? 1 : (units + 3) / 4);
+    if (x_dtype == VT_F32 && cache_dtype == VT_F32) qk_prepare_kernel<float, float><<<grid, 256, 0, stream>>>(a);
+    else if (x_dtype == VT_F32 && cache_dtype == VT_BF16) qk_prepare_kernel<float, bf16_t><<<grid, 256, 0, stream>>>(a);
+    else if (x_dtype == VT_BF16 && cache_dtype == VT_BF16) qk_prepare_kernel<bf16_t, bf16_t><<<grid, 256, 0, stream>>>(a);
     else return vt_fail("vt_qk_prepare: dtypes %d -> %d are not handled", x_dtype, cache_dtype);
     VT_CHECK_LAUNCH("vt_qk_prepare");
     return 0;

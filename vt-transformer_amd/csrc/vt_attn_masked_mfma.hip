@@ -3,7 +3,8 @@
 // is compiled: VT_KEY_DIM, VT_VALUE_DIM), one gate per head.
 //
 // A wave takes a tile of up to 16 consecutive tokens of one request and one query head; the host lists the tiles
-// (first row, rows).  Per 16 keys (one page, or part of one: pages hold a multiple of 16 keys):
+// (first row, rows).  A turn of the loop takes 32 keys, asked for a turn ahead.  Per 16 keys (one page, or part of one:
+// pages hold a multiple of 16 keys):
 //     S^T = K Q^T      [16 keys x 16 queries], v_mfma_f32_16x16x16 over the key size; A = K rows from the page
 //                      ([kv head][slot][D]: a lane reads 4 consecutive elements of its key), B = Q from registers
 //     cap, mask, running maximum and sum per query (a query is a column: its 16 scores lie in 4 lanes x 4 registers)
@@ -76,58 +77,99 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
     float m = -INFINITY, l = 0.f;
     const float nan = __int_as_float(0x7fc00000);
 
-    for (int kt = (lo / 16) * 16; kt <= pos_last; kt += 16) {
+    // Scores are kept times log2(e), so that every exponential is the hardware's 2^x.  The cap, with y = scale s / cap:
+    // cap tanh(y) = cap (1 - 2 / (1 + e^(2y))), e^(2y) = 2^(s c1).
+    const float LOG2E = 1.4426950408889634f;
+    const float c1 = a.cap > 0.f ? a.scale * 2.0f * LOG2E / a.cap : a.scale * LOG2E;
+    const float c2 = a.cap * LOG2E;
+    const int lo_last = [&] {
+        int v = a.chunk > 0 ? (pos_last / a.chunk) * a.chunk : 0;
+        if (a.window > 0) v = max(v, pos_last - a.window + 1);
+        return v;
+    }();
+
+    // 32 keys a turn, as two runs of 16 (each inside one page); a turn's keys and values are asked for a turn ahead
+    vt_lowp4_t kf[2][NK], vf[2][NV], kn[2][NK], vn[2][NV];
+    bool ok_now[2] = {false, false}, ok_next[2] = {false, false};
+    auto fetch = [&](int kt, vt_lowp4_t* kd, vt_lowp4_t* vd, bool& ok) {
         const int blk = kt / ps;
-        int pg = bt[blk];
-        const bool page_ok = pg >= 0 && pg < a.num_pages;
-        pg = page_ok ? pg : 0;
+        int pg = blk < a.max_blocks ? bt[blk] : -1;
+        ok = pg >= 0 && pg < a.num_pages;
+        pg = ok ? pg : 0;
         const int slot0 = kt - blk * ps;
         const bf16_t* kp = a.k_pages + (((size_t)pg * a.G + kvh) * ps + slot0 + r) * D + grp * 4;
         const bf16_t* vp = a.v_pages + (((size_t)pg * a.G + kvh) * DV + r) * ps + slot0 + grp * 4;
-        vt_lowp4_t kf[NK], vf[NV];
 #pragma unroll
-        for (int kk = 0; kk < NK; ++kk) kf[kk] = load4(kp + kk * 16);
+        for (int kk = 0; kk < NK; ++kk) kd[kk] = load4(kp + kk * 16);
 #pragma unroll
-        for (int v = 0; v < NV; ++v) vf[v] = load4(vp + (size_t)v * 16 * ps);
-        f32x4 s = {0.f, 0.f, 0.f, 0.f};
+        for (int v = 0; v < NV; ++v) vd[v] = load4(vp + (size_t)v * 16 * ps);
+    };
+    const int kt0 = (lo / 16) * 16;
+    fetch(kt0, kn[0], vn[0], ok_next[0]);
+    fetch(kt0 + 16, kn[1], vn[1], ok_next[1]);
+    for (int kt = kt0; kt <= pos_last; kt += 32) {
 #pragma unroll
-        for (int kk = 0; kk < NK; ++kk) s = VT_MFMA_16X16X16(kf[kk], qf[kk], s);
-        float sc[4];
-        float mt = -INFINITY;
+        for (int u = 0; u < 2; ++u) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int j = kt + grp * 4 + i;
-            float x = s[i] * a.scale;
-            if (a.cap > 0.f) {
-                // cap * tanh(x / cap), tanh(y) = 1 - 2 / (1 + e^(2y))
-                const float e = __expf(2.0f * x / a.cap);
-                x = a.cap * (1.0f - 2.0f / (1.0f + e));
-            }
-            const bool seen = row_ok && j <= pos && j >= lo_r;
-            x = seen ? (page_ok ? x : nan) : -INFINITY;      // a missing page must show, not pass as a masked key
-            sc[i] = x;
-            mt = fmaxf(mt, x);
+            for (int kk = 0; kk < NK; ++kk) kf[u][kk] = kn[u][kk];
+#pragma unroll
+            for (int v = 0; v < NV; ++v) vf[u][v] = vn[u][v];
+            ok_now[u] = ok_next[u];
         }
+        if (kt + 32 <= pos_last) {
+            fetch(kt + 32, kn[0], vn[0], ok_next[0]);
+            fetch(kt + 48, kn[1], vn[1], ok_next[1]);
+        }
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) {
+            s0 = VT_MFMA_16X16X16(kf[0][kk], qf[kk], s0);
+            s1 = VT_MFMA_16X16X16(kf[1][kk], qf[kk], s1);
+        }
+        float sc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float x = (i < 4 ? s0[i] : s1[i - 4]) * c1;
+            if (a.cap > 0.f) {
+                const float e = __builtin_amdgcn_exp2f(x);
+                sc[i] = fmaf(-2.0f * c2, __builtin_amdgcn_rcpf(1.0f + e), c2);
+            } else {
+                sc[i] = x;
+            }
+        }
+        // a turn that every row sees whole needs no mask
+        const bool whole = kt + 31 <= pos_first && kt >= lo_last && ok_now[0] && ok_now[1];
+        if (!whole) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int j = kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3);
+                const bool seen = row_ok && j <= pos && j >= lo_r;
+                // (a missing page must show, not pass as a masked key)
+                sc[i] = seen ? (ok_now[i >> 2] ? sc[i] : nan) : -INFINITY;
+            }
+        }
+        float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
         mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
         mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
         const float m_new = fmaxf(m, mt);
         const float mref = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = (m == -INFINITY) ? 0.f : __expf(m - m_new);
-        float p[4], psum = 0.f;
+        const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+        float p[8], psum = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            p[i] = __expf(sc[i] - mref);
+        for (int i = 0; i < 8; ++i) {
+            p[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
             psum += p[i];
         }
         l = l * alpha + psum;
         m = m_new;
-        const unsigned p01 = vt_pack2(p[0], p[1]), p23 = vt_pack2(p[2], p[3]);
-        struct { unsigned a, b; } pk = {p01, p23};
-        const vt_lowp4_t pf = __builtin_bit_cast(vt_lowp4_t, pk);
+        struct U2 { unsigned a, b; };
+        const U2 pk0 = {vt_pack2(p[0], p[1]), vt_pack2(p[2], p[3])}, pk1 = {vt_pack2(p[4], p[5]), vt_pack2(p[6], p[7])};
+        const vt_lowp4_t pf0 = __builtin_bit_cast(vt_lowp4_t, pk0), pf1 = __builtin_bit_cast(vt_lowp4_t, pk1);
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
             acc[v] *= alpha;
-            acc[v] = VT_MFMA_16X16X16(vf[v], pf, acc[v]);
+            acc[v] = VT_MFMA_16X16X16(vf[0][v], pf0, acc[v]);
+            acc[v] = VT_MFMA_16X16X16(vf[1][v], pf1, acc[v]);
         }
     }
     l += __shfl_xor(l, 16, 64);

@@ -128,14 +128,14 @@ extern "C" int vt_short_conv_carry(const void* x, int x_dtype, long long ldx, fl
 // ---------------------------------------------------------------------------
 struct DeltaArgs {
     const void* qkv;        // [n][C]: q (G x D), k (G x D), v (H x Dv), after convolution and SiLU
-    const float* ba;        // [n][2H]: beta logits, then decay logits
+    const void* ba;         // ba[t * ldba + h]: beta logits, then (from column H) decay logits
     const float* a_log;     // [H]
     const float* dt_bias;   // [H]
     float* state;           // slot s: state + s * slot_stride, [H][Dv][D]
     const int* entry_start;
     const int* slots;
     float* o;               // [n][H][Dv]
-    long long slot_stride;
+    long long slot_stride, ldba;
     int H, G, D, Dv;
 };
 
@@ -153,7 +153,10 @@ __device__ __forceinline__ float row16_sum(float v) {
 
 // DS: state elements per lane (a sixteenth of D, rounded up to a power of two).  Lane r of a column's 16 holds the
 // elements d = 16 i + r, i < DS: a row of lanes reads 16 consecutive floats of LDS or of the state at a time.
-template <typename TI, int DS>
+// The block's 256 threads are 16 columns x 16 lanes for the recurrence and 16 tokens x 16 lanes for a tile's inputs:
+// thread (tt, r) brings token tt's q and k elements 16 i + r, one of its values, and its gate and decay; a tile's
+// inputs are asked for from memory before the recurrence over the tile in front of it starts.
+template <typename TI, typename TB, int DS>
 __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
     constexpr int DP = 16 * DS;                       // D padded
     __shared__ float qs[DELTA_TILE][DP];
@@ -172,6 +175,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
     // the state of a head is kept [Dv][D]: a column's D elements lie together
     float* S_mem = a.state + (size_t)a.slots[e] * a.slot_stride + ((size_t)h * Dv + (col_ok ? col : 0)) * D;
     const TI* x = (const TI*)a.qkv;
+    const TB* ba = (const TB*)a.ba;
     const float decay_rate = expf(a.a_log[h]);
     const float bias = a.dt_bias[h];
     const float q_scale = 1.0f / sqrtf((float)D);
@@ -183,40 +187,52 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
         S[i] = (col_ok && d < D) ? S_mem[d] : 0.f;
     }
 
+    // a tile's inputs in registers, as thread (tt = cl, r) brings them
+    float in_q[DS], in_k[DS], in_v = 0.f, in_b = 0.f, in_a = 0.f;
+    auto fetch = [&](int t0) {
+        const int t = t0 + cl;
+        const bool ok = t < end;
+        const size_t row = (size_t)(ok ? t : start) * C;
+#pragma unroll
+        for (int i = 0; i < DS; ++i) {
+            const int d = 16 * i + r;
+            const bool in = ok && d < D;
+            in_q[i] = in ? load_f32<TI>(x, row + (size_t)kh * D + d) : 0.f;
+            in_k[i] = in ? load_f32<TI>(x, row + (size_t)(G + kh) * D + d) : 0.f;
+        }
+        in_v = (ok && col0 + r < Dv) ? load_f32<TI>(x, row + (size_t)2 * G * D + (size_t)h * Dv + col0 + r) : 0.f;
+        if (r == 0 && ok) {
+            in_b = load_f32<TB>(ba, (size_t)t * a.ldba + h);
+            in_a = load_f32<TB>(ba, (size_t)t * a.ldba + H + h);
+        }
+    };
+    fetch(start);
     for (int t0 = start; t0 < end; t0 += DELTA_TILE) {
         const int nt = min(DELTA_TILE, end - t0);
         __syncthreads();        // the tile before has been read
-        for (int i = tid; i < DELTA_TILE * DP; i += 256) {
-            const int tt = i / DP, d = i % DP;
-            float qv = 0.f, kv = 0.f;
-            if (tt < nt && d < D) {
-                const size_t row = (size_t)(t0 + tt) * C;
-                qv = load_f32<TI>(x, row + (size_t)kh * D + d);
-                kv = load_f32<TI>(x, row + (size_t)(G + kh) * D + d);
-            }
-            qs[tt][d] = qv;
-            ks[tt][d] = kv;
-        }
         {
-            const int tt = tid / DELTA_COLS, j = tid % DELTA_COLS;      // 16 tokens x 16 columns = the block's threads
-            vs[tt][j] = (tt < nt && col0 + j < Dv)
-                            ? load_f32<TI>(x, (size_t)(t0 + tt) * C + (size_t)2 * G * D + (size_t)h * Dv + col0 + j) : 0.f;
-        }
-        __syncthreads();
-        if (tid < nt) {
-            // lengths of q and k, gate and decay of one token, all in float32, sums in index order
+            // lengths of q and k (each lane's share, then the row's sum: the same order for every token), gate and
+            // decay of token cl, all in float32
             float sq = 0.f, sk = 0.f;
-            for (int d = 0; d < D; ++d) {
-                sq = fmaf(qs[tid][d], qs[tid][d], sq);
-                sk = fmaf(ks[tid][d], ks[tid][d], sk);
+#pragma unroll
+            for (int i = 0; i < DS; ++i) {
+                qs[cl][16 * i + r] = in_q[i];
+                ks[cl][16 * i + r] = in_k[i];
+                sq = fmaf(in_q[i], in_q[i], sq);
+                sk = fmaf(in_k[i], in_k[i], sk);
             }
-            rq_s[tid] = q_scale / sqrtf(sq + 1e-6f);
-            rk_s[tid] = 1.0f / sqrtf(sk + 1e-6f);
-            const float* ba = a.ba + (size_t)(t0 + tid) * 2 * H;
-            beta_s[tid] = 1.0f / (1.0f + expf(-ba[h]));
-            g_s[tid] = expf(-decay_rate * softplus_f(ba[H + h] + bias));
+            vs[cl][r] = in_v;
+            sq = row16_sum(sq);
+            sk = row16_sum(sk);
+            if (r == 0) {
+                rq_s[cl] = q_scale / sqrtf(sq + 1e-6f);
+                rk_s[cl] = 1.0f / sqrtf(sk + 1e-6f);
+                beta_s[cl] = 1.0f / (1.0f + expf(-in_b));
+                g_s[cl] = expf(-decay_rate * softplus_f(in_a + bias));
+            }
         }
         __syncthreads();
+        if (t0 + DELTA_TILE < end) fetch(t0 + DELTA_TILE);      // on its way while this tile is worked through
         for (int tt = 0; tt < nt; ++tt) {
             // with k' = rk k and q' = rq q:  S <- g S;  u = beta (v - k'.S);  S <- S + k' u;  o = q'.S
             const float g = g_s[tt], beta = beta_s[tt], rq = rq_s[tt], rk = rk_s[tt];
@@ -251,30 +267,32 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
     }
 }
 
-extern "C" int vt_delta_rule(const void* qkv, int dtype, const float* ba, const float* a_log, const float* dt_bias,
-                             float* state, long long slot_stride, const int* entry_start, const int* slots, float* o,
-                             int n_entries, int H, int G, int D, int Dv, hipStream_t stream) {
+extern "C" int vt_delta_rule(const void* qkv, int dtype, const void* ba, int ba_dtype, long long ldba, const float* a_log,
+                             const float* dt_bias, float* state, long long slot_stride, const int* entry_start,
+                             const int* slots, float* o, int n_entries, int H, int G, int D, int Dv, hipStream_t stream) {
     VT_REQUIRE(n_entries >= 0 && H > 0 && G > 0 && H % G == 0, "vt_delta_rule: bad heads %d/%d", H, G);
     VT_REQUIRE(D > 0 && D <= 256 && Dv > 0, "vt_delta_rule: head sizes %d/%d (keys up to 256)", D, Dv);
     VT_REQUIRE(slot_stride >= (long long)H * D * Dv, "vt_delta_rule: state slots are too short");
+    VT_REQUIRE(ldba >= 2 * H, "vt_delta_rule: rows of gate and decay logits are too short");
     VT_REQUIRE(H <= 65535, "vt_delta_rule: too many heads (%d)", H);
     if (n_entries == 0) return 0;
     DeltaArgs a;
     a.qkv = qkv; a.ba = ba; a.a_log = a_log; a.dt_bias = dt_bias; a.state = state; a.entry_start = entry_start;
-    a.slots = slots; a.o = o; a.slot_stride = slot_stride; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
+    a.slots = slots; a.o = o; a.slot_stride = slot_stride; a.ldba = ldba; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
     const dim3 grid(n_entries, H, (Dv + DELTA_COLS - 1) / DELTA_COLS);
     const int share = (D + 15) / 16;
-#define VT_DELTA(TI)                                                                          \
-    do {                                                                                      \
-        if (share <= 1) delta_rule_kernel<TI, 1><<<grid, 256, 0, stream>>>(a);                \
-        else if (share <= 2) delta_rule_kernel<TI, 2><<<grid, 256, 0, stream>>>(a);           \
-        else if (share <= 4) delta_rule_kernel<TI, 4><<<grid, 256, 0, stream>>>(a);           \
-        else if (share <= 8) delta_rule_kernel<TI, 8><<<grid, 256, 0, stream>>>(a);           \
-        else delta_rule_kernel<TI, 16><<<grid, 256, 0, stream>>>(a);                          \
+#define VT_DELTA(TI, TB)                                                                          \
+    do {                                                                                          \
+        if (share <= 1) delta_rule_kernel<TI, TB, 1><<<grid, 256, 0, stream>>>(a);                \
+        else if (share <= 2) delta_rule_kernel<TI, TB, 2><<<grid, 256, 0, stream>>>(a);           \
+        else if (share <= 4) delta_rule_kernel<TI, TB, 4><<<grid, 256, 0, stream>>>(a);           \
+        else if (share <= 8) delta_rule_kernel<TI, TB, 8><<<grid, 256, 0, stream>>>(a);           \
+        else delta_rule_kernel<TI, TB, 16><<<grid, 256, 0, stream>>>(a);                          \
     } while (0)
-    if (dtype == VT_F32) VT_DELTA(float);
-    else if (dtype == VT_BF16) VT_DELTA(bf16_t);
-    else return vt_fail("vt_delta_rule: unknown dtype %d", dtype);
+    if (dtype == VT_F32 && ba_dtype == VT_F32) VT_DELTA(float, float);
+    else if (dtype == VT_BF16 && ba_dtype == VT_F32) VT_DELTA(bf16_t, float);
+    else if (dtype == VT_BF16 && ba_dtype == VT_BF16) VT_DELTA(bf16_t, bf16_t);
+    else return vt_fail("vt_delta_rule: dtypes %d / %d are not handled", dtype, ba_dtype);
 #undef VT_DELTA
     VT_CHECK_LAUNCH("vt_delta_rule");
     return 0;

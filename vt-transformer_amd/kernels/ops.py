@@ -836,16 +836,21 @@ def short_conv_carry(x: torch.Tensor, channels: int, k: int, state: torch.Tensor
          sp, ss, _ptr(entry_start), _ptr(slots), _i(entry_start.numel() - 1), _i(channels), _i(k), _stream())
 
 
-def delta_rule(qkv: torch.Tensor, ba: torch.Tensor, a_log: torch.Tensor, dt_bias: torch.Tensor, state: torch.Tensor,
-               entry_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, key_dim: int,
-               value_dim: int) -> torch.Tensor:
+def delta_rule(qkv: torch.Tensor, ba: torch.Tensor, ba_column: int, a_log: torch.Tensor, dt_bias: torch.Tensor,
+               state: torch.Tensor, entry_start: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, n_heads: int,
+               n_kv: int, key_dim: int, value_dim: int) -> torch.Tensor:
     """The gated delta rule over the tokens of every entry, from and into state[slot] ([H, Dv, D] float32).
-    qkv [n, 2 G D + H Dv]: queries, keys (G heads of D), values (H heads of Dv); ba [n, 2 H] float32: logits of the
-    write strength and of the decay.  out [n, H * Dv] float32."""
+    qkv [n, 2 G D + H Dv]: queries, keys (G heads of D), values (H heads of Dv); ba: a 2-d tensor whose rows are the
+    tokens', with the H logits of the write strength from column ba_column and the H logits of the decay behind them
+    (float32, or the 16-bit type of qkv).  out [n, H * Dv] float32."""
     n = qkv.shape[0]
     c = 2 * n_kv * key_dim + n_heads * value_dim
     _chk(qkv, "delta_rule.qkv", None, (n, c))
-    _chk(ba, "delta_rule.ba", torch.float32, (n, 2 * n_heads))
+    _chk(ba, "delta_rule.ba")
+    if ba.dim() != 2 or ba.shape[0] != n or ba.shape[1] < ba_column + 2 * n_heads:
+        raise KernelError(f"delta_rule.ba: shape {tuple(ba.shape)} has no {2 * n_heads} columns from {ba_column}")
+    if ba.dtype != torch.float32 and ba.dtype != qkv.dtype:
+        raise KernelError(f"delta_rule: logits of dtype {ba.dtype} beside inputs of {qkv.dtype}")
     _chk(a_log, "delta_rule.a_log", torch.float32, (n_heads,))
     _chk(dt_bias, "delta_rule.dt_bias", torch.float32, (n_heads,))
     _chk(out, "delta_rule.out", torch.float32, (n, n_heads * value_dim))
@@ -854,9 +859,10 @@ def delta_rule(qkv: torch.Tensor, ba: torch.Tensor, a_log: torch.Tensor, dt_bias
     if key_dim > DELTA_MAX_KEY_DIM or n_heads % n_kv:
         raise KernelError(f"delta_rule: heads {n_heads}/{n_kv} of {key_dim}")
     sp, ss = _state_rows(state, "delta_rule", n_heads * key_dim * value_dim)
-    _run(load_lib("vt_delta", half=_half(qkv)), "vt_delta_rule", _ptr(qkv), _i(_code(qkv)), _ptr(ba), _ptr(a_log), _ptr(dt_bias),
-         sp, ss, _ptr(entry_start), _ptr(slots), _ptr(out), _i(entry_start.numel() - 1), _i(n_heads), _i(n_kv),
-         _i(key_dim), _i(value_dim), _stream())
+    bptr = ctypes.c_void_p(ba.data_ptr() + ba_column * ba.element_size())
+    _run(load_lib("vt_delta", half=_half(qkv, ba)), "vt_delta_rule", _ptr(qkv), _i(_code(qkv)), bptr, _i(_code(ba)),
+         ctypes.c_longlong(ba.stride(0)), _ptr(a_log), _ptr(dt_bias), sp, ss, _ptr(entry_start), _ptr(slots), _ptr(out),
+         _i(entry_start.numel() - 1), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _stream())
     return out
 
 

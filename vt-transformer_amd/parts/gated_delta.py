@@ -26,7 +26,7 @@ import torch
 
 from ..kernels import ops
 from .base import MIXERS, CacheNeed, Part, Runtime, StateNeed, TensorDecl
-from .linear import linear, linear_f32_out
+from .linear import linear
 
 
 @MIXERS.register("gated_delta")
@@ -60,7 +60,7 @@ class GatedDeltaMixer(Part):
         self.channels = 2 * self.nkv * self.d + self.nh * self.dv      # what the convolutions run over: q, k, v
         self.conv_floats = (self.taps - 1) * self.channels
         self.rule_floats = self.nh * self.d * self.dv
-        self.w_in = self.p_in = self.w_ba = self.p_ba = self.w_o = self.p_o = None
+        self.w_in = self.p_in = self.w_o = self.p_o = None
         self.conv_w = self.a_log = self.dt_bias = self.norm_w = None
 
     def cache_need(self) -> Optional[CacheNeed]:
@@ -93,13 +93,12 @@ class GatedDeltaMixer(Part):
 
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
         nm = self.names
-        self.w_in = torch.cat([rt.place(get(nm[k]), "matrix") for k in ("q", "k", "v", "g")], dim=0).contiguous()
-        self.w_ba = torch.cat([rt.place(get(nm[k]), "matrix") for k in ("b", "a")], dim=0).contiguous()
+        # one product for everything that reads the mixer's input: q, k, v, the output's gate, and the logits of the
+        # write strength and of the decay (what is computed from those two is float32)
+        self.w_in = torch.cat([rt.place(get(nm[k]), "matrix") for k in ("q", "k", "v", "g", "b", "a")], dim=0).contiguous()
         self.w_o = rt.place(get(nm["o"]), "matrix")
-        self.p_in, self.p_ba, self.p_o = rt.pack(self.w_in), rt.pack(self.w_ba), rt.pack(self.w_o)
+        self.p_in, self.p_o = rt.pack(self.w_in), rt.pack(self.w_o)
         self.w_in, self.w_o = rt.row_major(self.w_in, self.p_in), rt.row_major(self.w_o, self.p_o)
-        if self.p_ba is not None:
-            self.w_ba = None            # the small float32-output product always takes the packed copy
         if self.taps > 1:
             self.conv_w = torch.cat([rt.place(get(nm[k]), "bias") for k in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
         else:
@@ -113,14 +112,13 @@ class GatedDeltaMixer(Part):
         if state is None or state.dim() != 2 or state.shape[1] != self.conv_floats + self.rule_floats:
             raise RuntimeError("the gated delta mixer was given no state of its shape")
         conv_state, rule_state = state[:, :self.conv_floats], state[:, self.conv_floats:]
-        y = linear(rt, x, self.w_in, None, "delta.in", packed=self.p_in)            # q, k, v, gate
-        ba = linear_f32_out(rt, x, self.w_ba, None, "delta.ba", packed=self.p_ba)   # float32 at any number of rows
+        y = linear(rt, x, self.w_in, None, "delta.in", packed=self.p_in)            # q, k, v, gate, b, a
         qkv = rt.buffer("delta.qkv", (n, c), rt.dtype)
         ops.short_conv(y, c, self.conv_w, conv_state, ctx.tok_entry, ctx.entry_start, ctx.state_slots, qkv)
         if self.taps > 1:
             ops.short_conv_carry(y, c, self.taps, conv_state, ctx.entry_start, ctx.state_slots)
         o = rt.buffer("delta.o", (n, self.nh * self.dv), torch.float32)
-        ops.delta_rule(qkv, ba, self.a_log, self.dt_bias, rule_state, ctx.entry_start, ctx.state_slots, o, self.nh,
+        ops.delta_rule(qkv, y, c + self.nh * self.dv, self.a_log, self.dt_bias, rule_state, ctx.entry_start, ctx.state_slots, o, self.nh,
                        self.nkv, self.d, self.dv)
         z = rt.buffer("delta.gated", (n, self.nh * self.dv), rt.dtype)
         ops.gated_rmsnorm(o, self.norm_w, y, c, z, self.nh, self.dv, self.eps)

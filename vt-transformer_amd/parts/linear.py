@@ -139,22 +139,3 @@ def linear(rt: Runtime, x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.T
         torch.mm(x, w.t(), out=out)
     return out
 
-
-def linear_f32_out(rt: Runtime, x: torch.Tensor, w: Optional[torch.Tensor], bias: Optional[torch.Tensor], name: str,
-                   packed=None) -> torch.Tensor:
-    """x [N, K] -> float32 [N, M] at any number of rows: for the few products whose results must not be rounded to 16
-    bits on their way (logits of gates and decays that enter a recurrence).  In a 16-bit runtime the few-row kernel
-    takes the rows 64 at a time (it accumulates and stores in float32); meant for matrices with few rows, which
-    are then read once per 64 tokens."""
-    n, k = x.shape
-    m = w.shape[0] if w is not None else packed.rows
-    out = rt.buffer(name, (n, m), torch.float32)
-    if not rt.lowp:
-        return ops.linear_f32(x, w, bias, out)
-    wp = packed if packed is not None else w
-    for r0 in range(0, n, SKINNY_MAX_ROWS):
-        r1 = min(n, r0 + SKINNY_MAX_ROWS)
-        need = ops.linear_bf16_workspace(r1 - r0, m, k) if r1 - r0 > 16 else 0
-        work = rt.buffer("linear.partials", (need,), torch.float32) if need else None
-        ops.linear_bf16(x[r0:r1], wp, bias, out[r0:r1], work)
-    return out
