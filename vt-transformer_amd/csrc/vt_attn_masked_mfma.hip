@@ -88,15 +88,18 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
         return v;
     }();
 
-    // 32 keys a turn, as two runs of 16 (each inside one page); a turn's keys and values are asked for a turn ahead
+    // 32 keys a turn, as two runs of 16 (each inside one page).  A turn's keys and values are asked for a turn ahead,
+    // and the pages they lie in two turns ahead, so that no turn waits for a page number before it can ask for keys.
     vt_lowp4_t kf[2][NK], vf[2][NV], kn[2][NK], vn[2][NV];
     bool ok_now[2] = {false, false}, ok_next[2] = {false, false};
-    auto fetch = [&](int kt, vt_lowp4_t* kd, vt_lowp4_t* vd, bool& ok) {
+    auto page_of = [&](int kt) -> int {
         const int blk = kt / ps;
-        int pg = blk < a.max_blocks ? bt[blk] : -1;
+        return blk < a.max_blocks ? bt[blk] : -1;
+    };
+    auto fetch = [&](int kt, int pg, vt_lowp4_t* kd, vt_lowp4_t* vd, bool& ok) {
         ok = pg >= 0 && pg < a.num_pages;
         pg = ok ? pg : 0;
-        const int slot0 = kt - blk * ps;
+        const int slot0 = kt % ps;
         const bf16_t* kp = a.k_pages + (((size_t)pg * a.G + kvh) * ps + slot0 + r) * D + grp * 4;
         const bf16_t* vp = a.v_pages + (((size_t)pg * a.G + kvh) * DV + r) * ps + slot0 + grp * 4;
 #pragma unroll
@@ -105,8 +108,9 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
         for (int v = 0; v < NV; ++v) vd[v] = load4(vp + (size_t)v * 16 * ps);
     };
     const int kt0 = (lo / 16) * 16;
-    fetch(kt0, kn[0], vn[0], ok_next[0]);
-    fetch(kt0 + 16, kn[1], vn[1], ok_next[1]);
+    fetch(kt0, page_of(kt0), kn[0], vn[0], ok_next[0]);
+    fetch(kt0 + 16, page_of(kt0 + 16), kn[1], vn[1], ok_next[1]);
+    int pg_a = page_of(kt0 + 32), pg_b = page_of(kt0 + 48);
     for (int kt = kt0; kt <= pos_last; kt += 32) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -117,8 +121,10 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
             ok_now[u] = ok_next[u];
         }
         if (kt + 32 <= pos_last) {
-            fetch(kt + 32, kn[0], vn[0], ok_next[0]);
-            fetch(kt + 48, kn[1], vn[1], ok_next[1]);
+            fetch(kt + 32, pg_a, kn[0], vn[0], ok_next[0]);
+            fetch(kt + 48, pg_b, kn[1], vn[1], ok_next[1]);
+            pg_a = page_of(kt + 64);
+            pg_b = page_of(kt + 80);
         }
         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll

@@ -140,7 +140,7 @@ struct DeltaArgs {
 };
 
 #define DELTA_TILE 16
-#define DELTA_COLS 16
+#define DELTA_GROUPS 16     // column groups of a block: 16 lanes each
 
 // the sum of v over the 16 lanes of a row (lanes 16 r .. 16 r + 15), in every one of them: four rotations within the row
 __device__ __forceinline__ float row16_sum(float v) {
@@ -151,44 +151,50 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-// DS: state elements per lane (a sixteenth of D, rounded up to a power of two).  Lane r of a column's 16 holds the
-// elements d = 16 i + r, i < DS: a row of lanes reads 16 consecutive floats of LDS or of the state at a time.
-// The block's 256 threads are 16 columns x 16 lanes for the recurrence and 16 tokens x 16 lanes for a tile's inputs:
-// thread (tt, r) brings token tt's q and k elements 16 i + r, one of its values, and its gate and decay; a tile's
+// DS: state elements per lane and column (a sixteenth of D, rounded up to a power of two); CPL: columns per lane.
+// A row of 16 lanes shares CPL value columns; lane r holds the elements d = 16 i + r, i < DS, of each: a row reads 16
+// consecutive floats of LDS or of the state at a time, what it reads of k and q serves all its columns, and the
+// columns' sums are chains of additions that do not wait for each other.
+// The block's 256 threads are 16 rows of lanes for the recurrence and 16 tokens x 16 lanes for a tile's inputs:
+// thread (tt, r) brings token tt's q and k elements 16 i + r, CPL of its values, and its gate and decay; a tile's
 // inputs are asked for from memory before the recurrence over the tile in front of it starts.
-template <typename TI, typename TB, int DS>
+template <typename TI, typename TB, int DS, int CPL>
 __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
     constexpr int DP = 16 * DS;                       // D padded
+    constexpr int COLS = DELTA_GROUPS * CPL;          // columns of a block
     __shared__ float qs[DELTA_TILE][DP];
     __shared__ float ks[DELTA_TILE][DP];
-    __shared__ float vs[DELTA_TILE][DELTA_COLS];
+    __shared__ float vs[DELTA_TILE][COLS];
     __shared__ float beta_s[DELTA_TILE], g_s[DELTA_TILE], rq_s[DELTA_TILE], rk_s[DELTA_TILE];
 
-    const int e = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * DELTA_COLS;
+    const int e = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * COLS;
     const int tid = threadIdx.x;
-    const int r = tid & 15, cl = tid >> 4, col = col0 + cl;
-    const bool col_ok = col < a.Dv;
+    const int r = tid & 15, cl = tid >> 4;
     const int D = a.D, Dv = a.Dv, H = a.H, G = a.G;
     const int kh = h / (H / G);
     const int C = 2 * G * D + H * Dv;
     const int start = a.entry_start[e], end = a.entry_start[e + 1];
     // the state of a head is kept [Dv][D]: a column's D elements lie together
-    float* S_mem = a.state + (size_t)a.slots[e] * a.slot_stride + ((size_t)h * Dv + (col_ok ? col : 0)) * D;
+    float* S_head = a.state + (size_t)a.slots[e] * a.slot_stride + (size_t)h * Dv * D;
     const TI* x = (const TI*)a.qkv;
     const TB* ba = (const TB*)a.ba;
     const float decay_rate = expf(a.a_log[h]);
     const float bias = a.dt_bias[h];
     const float q_scale = 1.0f / sqrtf((float)D);
 
-    float S[DS];
+    float S[CPL][DS];
 #pragma unroll
-    for (int i = 0; i < DS; ++i) {
-        const int d = 16 * i + r;
-        S[i] = (col_ok && d < D) ? S_mem[d] : 0.f;
+    for (int c = 0; c < CPL; ++c) {
+        const int col = col0 + cl * CPL + c;
+#pragma unroll
+        for (int i = 0; i < DS; ++i) {
+            const int d = 16 * i + r;
+            S[c][i] = (col < Dv && d < D) ? S_head[(size_t)col * D + d] : 0.f;
+        }
     }
 
     // a tile's inputs in registers, as thread (tt = cl, r) brings them
-    float in_q[DS], in_k[DS], in_v = 0.f, in_b = 0.f, in_a = 0.f;
+    float in_q[DS], in_k[DS], in_v[CPL], in_b = 0.f, in_a = 0.f;
     auto fetch = [&](int t0) {
         const int t = t0 + cl;
         const bool ok = t < end;
@@ -200,7 +206,11 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
             in_q[i] = in ? load_f32<TI>(x, row + (size_t)kh * D + d) : 0.f;
             in_k[i] = in ? load_f32<TI>(x, row + (size_t)(G + kh) * D + d) : 0.f;
         }
-        in_v = (ok && col0 + r < Dv) ? load_f32<TI>(x, row + (size_t)2 * G * D + (size_t)h * Dv + col0 + r) : 0.f;
+#pragma unroll
+        for (int c = 0; c < CPL; ++c) {
+            const int j = col0 + r * CPL + c;
+            in_v[c] = (ok && j < Dv) ? load_f32<TI>(x, row + (size_t)2 * G * D + (size_t)h * Dv + j) : 0.f;
+        }
         if (r == 0 && ok) {
             in_b = load_f32<TB>(ba, (size_t)t * a.ldba + h);
             in_a = load_f32<TB>(ba, (size_t)t * a.ldba + H + h);
@@ -221,7 +231,8 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
                 sq = fmaf(in_q[i], in_q[i], sq);
                 sk = fmaf(in_k[i], in_k[i], sk);
             }
-            vs[cl][r] = in_v;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) vs[cl][r * CPL + c] = in_v[c];
             sq = row16_sum(sq);
             sk = row16_sum(sk);
             if (r == 0) {
@@ -233,8 +244,8 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
         }
         __syncthreads();
         if (t0 + DELTA_TILE < end) fetch(t0 + DELTA_TILE);      // on its way while this tile is worked through
+        // with k' = rk k and q' = rq q:  S <- g S;  u = beta (v - k'.S);  S <- S + k' u;  o = q'.S
         for (int tt = 0; tt < nt; ++tt) {
-            // with k' = rk k and q' = rq q:  S <- g S;  u = beta (v - k'.S);  S <- S + k' u;  o = q'.S
             const float g = g_s[tt], beta = beta_s[tt], rq = rq_s[tt], rk = rk_s[tt];
             float kk[DS], qq[DS];
 #pragma unroll
@@ -242,28 +253,50 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
                 kk[i] = ks[tt][16 * i + r];
                 qq[i] = qs[tt][16 * i + r];
             }
-            float dot = 0.f;
+            float dot[CPL], out[CPL];
 #pragma unroll
-            for (int i = 0; i < DS; ++i) {
-                S[i] *= g;
-                dot = fmaf(kk[i], S[i], dot);
-            }
-            dot = row16_sum(dot);
-            const float u = beta * (vs[tt][cl] - rk * dot) * rk;
-            float out = 0.f;
+            for (int c = 0; c < CPL; ++c) {
+                float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < DS; ++i) {
-                S[i] = fmaf(kk[i], u, S[i]);
-                out = fmaf(qq[i], S[i], out);
+                for (int i = 0; i < DS; ++i) {
+                    S[c][i] *= g;
+                    acc = fmaf(kk[i], S[c][i], acc);
+                }
+                dot[c] = acc;
             }
-            out = row16_sum(out);
-            if (r == 0 && col_ok) a.o[((size_t)(t0 + tt) * H + h) * Dv + col] = rq * out;
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) dot[c] = row16_sum(dot[c]);
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) {
+                const float u = beta * (vs[tt][cl * CPL + c] - rk * dot[c]) * rk;
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < DS; ++i) {
+                    S[c][i] = fmaf(kk[i], u, S[c][i]);
+                    acc = fmaf(qq[i], S[c][i], acc);
+                }
+                out[c] = acc;
+            }
+#pragma unroll
+            for (int c = 0; c < CPL; ++c) out[c] = row16_sum(out[c]);
+            if (r == 0) {
+                float* o = a.o + ((size_t)(t0 + tt) * H + h) * Dv;
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) {
+                    const int col = col0 + cl * CPL + c;
+                    if (col < Dv) o[col] = rq * out[c];
+                }
+            }
         }
     }
 #pragma unroll
-    for (int i = 0; i < DS; ++i) {
-        const int d = 16 * i + r;
-        if (col_ok && d < D) S_mem[d] = S[i];
+    for (int c = 0; c < CPL; ++c) {
+        const int col = col0 + cl * CPL + c;
+#pragma unroll
+        for (int i = 0; i < DS; ++i) {
+            const int d = 16 * i + r;
+            if (col < Dv && d < D) S_head[(size_t)col * D + d] = S[c][i];
+        }
     }
 }
 
@@ -279,15 +312,20 @@ extern "C" int vt_delta_rule(const void* qkv, int dtype, const void* ba, int ba_
     DeltaArgs a;
     a.qkv = qkv; a.ba = ba; a.a_log = a_log; a.dt_bias = dt_bias; a.state = state; a.entry_start = entry_start;
     a.slots = slots; a.o = o; a.slot_stride = slot_stride; a.ldba = ldba; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
-    const dim3 grid(n_entries, H, (Dv + DELTA_COLS - 1) / DELTA_COLS);
+    // One column to a row of lanes.  (The kernel also takes CPL = 4, four columns to a row, which shares what a row
+    // reads of k and q among them; measured at 16 heads of 128 x 128 it was no faster with eight requests and half
+    // again slower with one: a lone wave per SIMD issues its longer stream no faster.)
+    constexpr int cpl = 1;
     const int share = (D + 15) / 16;
-#define VT_DELTA(TI, TB)                                                                          \
-    do {                                                                                          \
-        if (share <= 1) delta_rule_kernel<TI, TB, 1><<<grid, 256, 0, stream>>>(a);                \
-        else if (share <= 2) delta_rule_kernel<TI, TB, 2><<<grid, 256, 0, stream>>>(a);           \
-        else if (share <= 4) delta_rule_kernel<TI, TB, 4><<<grid, 256, 0, stream>>>(a);           \
-        else if (share <= 8) delta_rule_kernel<TI, TB, 8><<<grid, 256, 0, stream>>>(a);           \
-        else delta_rule_kernel<TI, TB, 16><<<grid, 256, 0, stream>>>(a);                          \
+    const int cols = DELTA_GROUPS * cpl;
+    const dim3 grid(n_entries, H, (Dv + cols - 1) / cols);
+#define VT_DELTA(TI, TB)                                                                           \
+    do {                                                                                           \
+        if (share <= 1) delta_rule_kernel<TI, TB, 1, cpl><<<grid, 256, 0, stream>>>(a);            \
+        else if (share <= 2) delta_rule_kernel<TI, TB, 2, cpl><<<grid, 256, 0, stream>>>(a);       \
+        else if (share <= 4) delta_rule_kernel<TI, TB, 4, cpl><<<grid, 256, 0, stream>>>(a);       \
+        else if (share <= 8) delta_rule_kernel<TI, TB, 8, cpl><<<grid, 256, 0, stream>>>(a);       \
+        else delta_rule_kernel<TI, TB, 16, cpl><<<grid, 256, 0, stream>>>(a);                      \
     } while (0)
     if (dtype == VT_F32 && ba_dtype == VT_F32) VT_DELTA(float, float);
     else if (dtype == VT_BF16 && ba_dtype == VT_F32) VT_DELTA(bf16_t, float);
