@@ -103,7 +103,7 @@ def test_embedding_scale_and_stream_offsets():
     (3, 3, 16, 16, 16, 7, 0, 0.0, False, False),     # whole head rotated, nothing else but the chunks
     (6, 1, 40, 24, 0, 0, 0, 5.0, True, True),        # no rotation, every earlier key
     (2, 1, 24, 136, 12, 50, 20, 0.0, True, False),   # window inside chunks, values larger than keys
-    (2, 1, 64, 80, 16, 50, 20, 10.0, True, True),    # the same on the matrix cores (heads in multiples of 16)
+    (2, 1, 64, 96, 16, 50, 20, 10.0, True, True),    # the same on the matrix cores (heads in multiples of 16)
 ])
 def test_masked_attention_part(dtype, nh, kvh, d, dv, rot, chunk, window, cap, gate, unit):
     from vt_transformer_amd.engine.step import ModelRunner

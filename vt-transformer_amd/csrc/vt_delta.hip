@@ -245,7 +245,7 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
         __syncthreads();
         if (t0 + DELTA_TILE < end) fetch(t0 + DELTA_TILE);      // on its way while this tile is worked through
         // with k' = rk k and q' = rq q:  S <- g S;  u = beta (v - k'.S);  S <- S + k' u;  o = q'.S
-        for (int tt = 0; tt < nt; ++tt) {
+        auto token = [&](int tt) {
             const float g = g_s[tt], beta = beta_s[tt], rq = rq_s[tt], rk = rk_s[tt];
             float kk[DS], qq[DS];
 #pragma unroll
@@ -287,6 +287,14 @@ __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs a) {
                     if (col < Dv) o[col] = rq * out[c];
                 }
             }
+        };
+        if (nt == DELTA_TILE) {
+            // a whole tile as one stretch of code: a token's read-out and the next token's sums do not wait for each
+            // other, and what they read from LDS is asked for early
+#pragma unroll
+            for (int tt = 0; tt < DELTA_TILE; ++tt) token(tt);
+        } else {
+            for (int tt = 0; tt < nt; ++tt) token(tt);
         }
     }
 #pragma unroll
