@@ -104,6 +104,8 @@ def test_embedding_scale_and_stream_offsets():
     (6, 1, 40, 24, 0, 0, 0, 5.0, True, True),        # no rotation, every earlier key
     (2, 1, 24, 136, 12, 50, 20, 0.0, True, False),   # window inside chunks, values larger than keys
     (2, 1, 64, 96, 16, 50, 20, 10.0, True, True),    # the same on the matrix cores (heads in multiples of 16)
+    (8, 2, 32, 48, 8, 24, 0, 15.0, True, True),      # four query heads to a key/value head: a block's waves share keys
+    (4, 1, 16, 16, 16, 7, 11, 0.0, False, True),     # ... with a window inside small chunks
 ])
 def test_masked_attention_part(dtype, nh, kvh, d, dv, rot, chunk, window, cap, gate, unit):
     from vt_transformer_amd.engine.step import ModelRunner
@@ -169,7 +171,7 @@ def test_one_key_that_stands_out_at_chunk_and_page_edges(dtype, matrix):
     from vt_transformer_amd.kernels import ops
     from vt_transformer_amd.parts import MIXERS
     rt = runtime(dtype)
-    nh, kvh, d, dv, chunk = 2, 1, 16, 16, 320
+    nh, kvh, d, dv, chunk = (4 if matrix else 2), 1, 16, 16, 320      # (four heads to a key/value head: the kernel whose waves share keys)
     mixer = MIXERS.build(PartSpec("masked_attention", dict(num_heads=nh, num_kv_heads=kvh, key_dim=d, value_dim=dv,
                                                            scale=1.0, chunk=chunk)), rt=rt, width=8, prefix="a.", shared={})
     runner = ModelRunner(OneMixer(mixer), rt, 16, 1024, 2, 1024)
@@ -177,8 +179,8 @@ def test_one_key_that_stands_out_at_chunk_and_page_edges(dtype, matrix):
     g = torch.Generator().manual_seed(5)
     y = torch.randn(t, (nh + kvh) * d + kvh * dv, generator=g) * 0.1
     y[:, :nh * d] = 0
-    y[:, 0] = 6.0                          # every query points along element 0 ...
-    y[:, d] = 6.0
+    for hh in range(nh):
+        y[:, hh * d] = 6.0                 # every query points along element 0 ...
     y[star, nh * d] = 6.0                  # ... and so does the one key: score 36 against about 0
     y[star, (nh + kvh) * d:] = 50.0
     far = chunk - 1                        # the last position that sees it

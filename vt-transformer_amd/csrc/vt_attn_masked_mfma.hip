@@ -196,6 +196,196 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
     }
 }
 
+// The same work with the block's four waves sharing what they read: when a key/value head serves a multiple of four
+// query heads, the four waves of a block are four heads of one group on the same 16 tokens, so they want the same keys
+// and values.  The block brings a turn's 32 keys and their values from the pages once (every thread a few 16-byte
+// pieces, a turn ahead, into registers), puts them into LDS (two buffers, rows padded against bank conflicts: one
+// barrier a turn), and every wave reads its matrix operands from there.
+__global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a) {
+    constexpr int D = VT_KEY_DIM, DV = VT_VALUE_DIM, NK = D / 16, NV = DV / 16;
+    constexpr int KROW = D + 4;                 // elements of a key's row in LDS
+    constexpr int VROW = 32 + 4;                // elements of a value element's row in LDS: 32 keys
+    constexpr int KP = (4 * D + 255) / 256;     // 16-byte pieces of a turn's keys per thread
+    constexpr int VP = (4 * DV + 255) / 256;    // ... of its values
+    __shared__ __attribute__((aligned(16))) bf16_t k_lds[2][32 * KROW];
+    __shared__ __attribute__((aligned(16))) bf16_t v_lds[2][DV * VROW];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int item = blockIdx.x * 4 + (tid >> 6);       // (the launch has whole blocks: the heads are a multiple of four)
+    const int tile = item / a.H, h = item % a.H;
+    const int kvh = h / (a.H / a.G);
+    const int first = a.tiles[2 * tile], rows = a.tiles[2 * tile + 1];
+    const int r = lane & 15, grp = lane >> 4;
+    const bool row_ok = r < rows;
+    const int t = first + (row_ok ? r : 0);
+    const int pos = a.positions[t];
+    const int pos_first = a.positions[first], pos_last = a.positions[first + rows - 1];
+    const int* bt = a.block_table + (size_t)a.tok_entry[first] * a.max_blocks;
+    const int ps = a.page_size;
+
+    int lo_r = a.chunk > 0 ? (pos / a.chunk) * a.chunk : 0;
+    if (a.window > 0) lo_r = max(lo_r, pos - a.window + 1);
+    int lo = a.chunk > 0 ? (pos_first / a.chunk) * a.chunk : 0;
+    if (a.window > 0) lo = max(lo, pos_first - a.window + 1);
+    int lo_last = a.chunk > 0 ? (pos_last / a.chunk) * a.chunk : 0;
+    if (a.window > 0) lo_last = max(lo_last, pos_last - a.window + 1);
+
+    vt_lowp4_t qf[NK];
+    {
+        const bf16_t* qr = a.q + ((size_t)t * a.H + h) * D + grp * 4;
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) {
+            qf[kk] = load4(qr + kk * 16);
+            if (!row_ok) qf[kk] = (vt_lowp4_t){0, 0, 0, 0};
+        }
+    }
+    f32x4 acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const float nan = __int_as_float(0x7fc00000);
+    const float LOG2E = 1.4426950408889634f;
+    const float c1 = a.cap > 0.f ? a.scale * 2.0f * LOG2E / a.cap : a.scale * LOG2E;
+    const float c2 = a.cap * LOG2E;
+
+    auto page_of = [&](int kt) -> int {
+        const int blk = kt / ps;
+        return blk < a.max_blocks ? bt[blk] : -1;
+    };
+    uint4 kreg[KP], vreg[VP];
+    bool ok_next[2] = {false, false}, ok_now[2] = {false, false};
+    auto fetch = [&](int kt, int pg0, int pg1) {
+        ok_next[0] = pg0 >= 0 && pg0 < a.num_pages;
+        ok_next[1] = pg1 >= 0 && pg1 < a.num_pages;
+        const size_t base0 = ((size_t)(ok_next[0] ? pg0 : 0) * a.G + kvh), base1 = ((size_t)(ok_next[1] ? pg1 : 0) * a.G + kvh);
+        const int slot_a = kt % ps, slot_b = (kt + 16) % ps;
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int p = tid + 256 * i;
+            if (p < 4 * D) {
+                const int key = p / (D / 8), off = (p % (D / 8)) * 8;
+                const bf16_t* src = a.k_pages + ((key < 16 ? base0 : base1) * ps + (key < 16 ? slot_a + key : slot_b + key - 16)) * D + off;
+                kreg[i] = *(const uint4*)src;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int p = tid + 256 * i;
+            if (p < 4 * DV) {
+                const int row = p >> 2, q4 = p & 3;
+                const bf16_t* src = a.v_pages + ((q4 < 2 ? base0 : base1) * DV + row) * ps + (q4 < 2 ? slot_a : slot_b) + (q4 & 1) * 8;
+                vreg[i] = *(const uint4*)src;
+            }
+        }
+    };
+    auto to_lds = [&](int b) {
+#pragma unroll
+        for (int i = 0; i < KP; ++i) {
+            const int p = tid + 256 * i;
+            if (p < 4 * D) {
+                const int key = p / (D / 8), off = (p % (D / 8)) * 8;
+                uint2* dst = (uint2*)&k_lds[b][key * KROW + off];
+                dst[0] = make_uint2(kreg[i].x, kreg[i].y);
+                dst[1] = make_uint2(kreg[i].z, kreg[i].w);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < VP; ++i) {
+            const int p = tid + 256 * i;
+            if (p < 4 * DV) {
+                const int row = p >> 2, q4 = p & 3;
+                uint2* dst = (uint2*)&v_lds[b][row * VROW + q4 * 8];
+                dst[0] = make_uint2(vreg[i].x, vreg[i].y);
+                dst[1] = make_uint2(vreg[i].z, vreg[i].w);
+            }
+        }
+    };
+
+    const int kt0 = (lo / 16) * 16;
+    fetch(kt0, page_of(kt0), page_of(kt0 + 16));
+    int pg_a = page_of(kt0 + 32), pg_b = page_of(kt0 + 48);
+    int b = 0;
+    for (int kt = kt0; kt <= pos_last; kt += 32) {
+        to_lds(b);
+        ok_now[0] = ok_next[0];
+        ok_now[1] = ok_next[1];
+        if (kt + 32 <= pos_last) {
+            fetch(kt + 32, pg_a, pg_b);
+            pg_a = page_of(kt + 64);
+            pg_b = page_of(kt + 80);
+        }
+        __syncthreads();
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+        const bf16_t* kl = &k_lds[b][r * KROW + grp * 4];
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) {
+            s0 = VT_MFMA_16X16X16(load4(kl + kk * 16), qf[kk], s0);
+            s1 = VT_MFMA_16X16X16(load4(kl + 16 * KROW + kk * 16), qf[kk], s1);
+        }
+        float sc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float x = (i < 4 ? s0[i] : s1[i - 4]) * c1;
+            if (a.cap > 0.f) {
+                const float e = __builtin_amdgcn_exp2f(x);
+                sc[i] = fmaf(-2.0f * c2, __builtin_amdgcn_rcpf(1.0f + e), c2);
+            } else {
+                sc[i] = x;
+            }
+        }
+        const bool whole = kt + 31 <= pos_first && kt >= lo_last && ok_now[0] && ok_now[1];
+        if (!whole) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int j = kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3);
+                const bool seen = row_ok && j <= pos && j >= lo_r;
+                sc[i] = seen ? (ok_now[i >> 2] ? sc[i] : nan) : -INFINITY;
+            }
+        }
+        float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m, mt);
+        const float mref = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+        float p[8], psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            p[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
+            psum += p[i];
+        }
+        l = l * alpha + psum;
+        m = m_new;
+        struct U2 { unsigned a, b; };
+        const U2 pk0 = {vt_pack2(p[0], p[1]), vt_pack2(p[2], p[3])}, pk1 = {vt_pack2(p[4], p[5]), vt_pack2(p[6], p[7])};
+        const vt_lowp4_t pf0 = __builtin_bit_cast(vt_lowp4_t, pk0), pf1 = __builtin_bit_cast(vt_lowp4_t, pk1);
+        const bf16_t* vl = &v_lds[b][r * VROW + grp * 4];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            acc[v] *= alpha;
+            acc[v] = VT_MFMA_16X16X16(load4(vl + v * 16 * VROW), pf0, acc[v]);
+            acc[v] = VT_MFMA_16X16X16(load4(vl + v * 16 * VROW + 16), pf1, acc[v]);
+        }
+        b ^= 1;
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!row_ok) return;
+    float gate = 1.f;
+    if (a.gate) {
+        const size_t gi = (size_t)t * a.ldg + h;
+        const float z = a.gate_f32 ? ((const float*)a.gate)[gi] : bf16_to_f32(((const bf16_t*)a.gate)[gi]);
+        gate = 1.0f / (1.0f + expf(-z));
+    }
+    const float f = gate / l;
+    bf16_t* o = a.out + ((size_t)t * a.H + h) * DV + grp * 4;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+        struct { unsigned a, b; } ok = {vt_pack2(acc[v][0] * f, acc[v][1] * f), vt_pack2(acc[v][2] * f, acc[v][3] * f)};
+        *(uint2*)(o + v * 16) = __builtin_bit_cast(uint2, ok);
+    }
+}
+
 extern "C" int vt_attn_masked_mfma_dims(int* key_dim, int* value_dim) {
     *key_dim = VT_KEY_DIM;
     *value_dim = VT_VALUE_DIM;
@@ -221,7 +411,10 @@ extern "C" int vt_attn_masked_mfma(const void* q, const void* k_pages, const voi
     a.n_tiles = n_tiles; a.H = H; a.G = G; a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages;
     a.window = window; a.chunk = chunk; a.gate_f32 = gate_dtype == VT_F32; a.scale = scale; a.cap = cap;
     const long long items = (long long)n_tiles * H;
-    attn_masked_mfma_kernel<<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(a);
+    if ((H / G) % 4 == 0)       // four heads of one key/value group to a block: they share what they read
+        attn_masked_mfma_shared_kernel<<<(unsigned)(items / 4), 256, 0, stream>>>(a);
+    else
+        attn_masked_mfma_kernel<<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_masked_mfma");
     return 0;
 }
