@@ -98,3 +98,23 @@ def test_stretched_frequencies_of_the_rotary_part():
     ang = torch.arange(64, dtype=pl.DT)[:, None] * f[None, :]
     assert float((torch.from_numpy(cos).double() - torch.cos(ang) * mag).abs().max()) < 1e-7
     assert float((torch.from_numpy(sin).double() - torch.sin(ang) * mag).abs().max()) < 1e-7
+
+
+def test_random_model_through_the_command_line(tmp_path):
+    """`--write-random-model` with a Lisunex config.json: the folder holds the configuration back and every tensor the
+    model declares, and the plain implementation runs it."""
+    import json
+    import subprocess
+    import sys
+    from replay_helpers import ROOT
+    cfg_path = tmp_path / "cfg.json"
+    cfg_path.write_text(json.dumps(CONFIGS["C"]))
+    out = tmp_path / "model"
+    r = subprocess.run([sys.executable, "-m", "vt_transformer_amd", "--write-random-model", str(out), "--config", str(cfg_path),
+                        "--seed", "5"], cwd=ROOT, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    cfg, w = pl.read_folder(str(out))
+    assert cfg["architecture"] == "Lisunex" and cfg["loop"] == CONFIGS["C"]["loop"] and cfg["layers"] == CONFIGS["C"]["layers"]
+    assert set(w) == set(declared_tensors(config_from_dict(copy.deepcopy(CONFIGS["C"]))))
+    logits = pl.forward(cfg, w, [3, 1, 4, 1, 5, 9, 2, 6])
+    assert logits.shape == (8, CONFIGS["C"]["vocab"]) and bool(torch.isfinite(logits).all())

@@ -202,8 +202,10 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
 // pieces, a turn ahead, into registers), puts them into LDS (two buffers, rows padded against bank conflicts: one
 // barrier a turn), and every wave reads its matrix operands from there.
 __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a) {
-    constexpr int D = VT_KEY_DIM, DV = VT_VALUE_DIM, NK = D / 16, NV = DV / 16;
-    constexpr int KROW = D + 4;                 // elements of a key's row in LDS
+    constexpr int D = VT_KEY_DIM, DV = VT_VALUE_DIM, NV = DV / 16;
+    constexpr int NK32 = D / 32;                // products of 32 key elements; a key size that is no multiple of 32 ends in one of 16
+    constexpr bool TAIL = D % 32 != 0;
+    constexpr int KROW = D + 8;                 // elements of a key's row in LDS (rows stay 16-byte aligned)
     constexpr int VROW = 32 + 4;                // elements of a value element's row in LDS: 32 keys
     constexpr int KP = (4 * D + 255) / 256;     // 16-byte pieces of a turn's keys per thread
     constexpr int VP = (4 * DV + 255) / 256;    // ... of its values
@@ -230,14 +232,18 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
     int lo_last = a.chunk > 0 ? (pos_last / a.chunk) * a.chunk : 0;
     if (a.window > 0) lo_last = max(lo_last, pos_last - a.window + 1);
 
-    vt_lowp4_t qf[NK];
+    // queries as the second operand of v_mfma_f32_16x16x32: a lane holds 8 consecutive elements of its row
+    vt_lowp8_t qf[NK32 > 0 ? NK32 : 1];
+    vt_lowp4_t qtail = {0, 0, 0, 0};
     {
-        const bf16_t* qr = a.q + ((size_t)t * a.H + h) * D + grp * 4;
+        const bf16_t* qrow = a.q + ((size_t)t * a.H + h) * D;
+        const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
-        for (int kk = 0; kk < NK; ++kk) {
-            qf[kk] = load4(qr + kk * 16);
-            if (!row_ok) qf[kk] = (vt_lowp4_t){0, 0, 0, 0};
+        for (int kk = 0; kk < NK32; ++kk) {
+            const uint4 raw = row_ok ? *(const uint4*)(qrow + kk * 32 + grp * 8) : zero4;
+            qf[kk] = __builtin_bit_cast(vt_lowp8_t, raw);
         }
+        if (TAIL && row_ok) qtail = load4(qrow + (D - 16) + grp * 4);
     }
     f32x4 acc[NV];
 #pragma unroll
@@ -316,11 +322,17 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
         }
         __syncthreads();
         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
-        const bf16_t* kl = &k_lds[b][r * KROW + grp * 4];
+        const bf16_t* kl = &k_lds[b][r * KROW];
 #pragma unroll
-        for (int kk = 0; kk < NK; ++kk) {
-            s0 = VT_MFMA_16X16X16(load4(kl + kk * 16), qf[kk], s0);
-            s1 = VT_MFMA_16X16X16(load4(kl + 16 * KROW + kk * 16), qf[kk], s1);
+        for (int kk = 0; kk < NK32; ++kk) {
+            const vt_lowp8_t k0 = __builtin_bit_cast(vt_lowp8_t, *(const uint4*)(kl + kk * 32 + grp * 8));
+            const vt_lowp8_t k1 = __builtin_bit_cast(vt_lowp8_t, *(const uint4*)(kl + 16 * KROW + kk * 32 + grp * 8));
+            s0 = VT_MFMA_16X16X32(k0, qf[kk], s0);
+            s1 = VT_MFMA_16X16X32(k1, qf[kk], s1);
+        }
+        if (TAIL) {
+            s0 = VT_MFMA_16X16X16(load4(kl + (D - 16) + grp * 4), qtail, s0);
+            s1 = VT_MFMA_16X16X16(load4(kl + 16 * KROW + (D - 16) + grp * 4), qtail, s1);
         }
         float sc[8];
 #pragma unroll
@@ -356,15 +368,18 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
         }
         l = l * alpha + psum;
         m = m_new;
-        struct U2 { unsigned a, b; };
-        const U2 pk0 = {vt_pack2(p[0], p[1]), vt_pack2(p[2], p[3])}, pk1 = {vt_pack2(p[4], p[5]), vt_pack2(p[6], p[7])};
-        const vt_lowp4_t pf0 = __builtin_bit_cast(vt_lowp4_t, pk0), pf1 = __builtin_bit_cast(vt_lowp4_t, pk1);
+        // One product over the turn's 32 keys.  Its key index 8 grp + j stands for key 4 grp + j of the first run
+        // (j < 4) and key 16 + 4 grp + j - 4 of the second: that is the order of the lane's eight probabilities, and the
+        // values are read from LDS in the same order.
+        const uint4 praw = make_uint4(vt_pack2(p[0], p[1]), vt_pack2(p[2], p[3]), vt_pack2(p[4], p[5]), vt_pack2(p[6], p[7]));
+        const vt_lowp8_t pf = __builtin_bit_cast(vt_lowp8_t, praw);
         const bf16_t* vl = &v_lds[b][r * VROW + grp * 4];
 #pragma unroll
         for (int v = 0; v < NV; ++v) {
+            const uint2 va = *(const uint2*)(vl + v * 16 * VROW), vb = *(const uint2*)(vl + v * 16 * VROW + 16);
+            const vt_lowp8_t vf = __builtin_bit_cast(vt_lowp8_t, make_uint4(va.x, va.y, vb.x, vb.y));
             acc[v] *= alpha;
-            acc[v] = VT_MFMA_16X16X16(load4(vl + v * 16 * VROW), pf0, acc[v]);
-            acc[v] = VT_MFMA_16X16X16(load4(vl + v * 16 * VROW + 16), pf1, acc[v]);
+            acc[v] = VT_MFMA_16X16X32(vf, pf, acc[v]);
         }
         b ^= 1;
     }
