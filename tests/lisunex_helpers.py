@@ -16,7 +16,7 @@ import plain_lisunex as pl
 # bfloat16 rounds every activation to eight bits, about 4e-3 each, through up to seven layer runs of these weights; a
 # portion of more than 64 tokens also gets its projections' results in 16 bits (the GEMM library's), the logits of the
 # delta rule's decay among them, which these weights make steep
-TOL = {"float32": 3e-5, "bfloat16": 4e-2}
+TOL = {"float32": 3e-5, "bfloat16": 3e-2}
 
 
 def attention_layer(heads=4, kv_heads=2, dim=32, vdim=48, scale=0.2, softcap=15.0, chunk=24, rot_dims=8, base=10000.0,
@@ -109,7 +109,7 @@ def check_logits(model_dir: str, reqs: Dict[str, List[int]], steps: List[dict], 
             cache[key] = pl.forward(cfg, w, toks).numpy()
         ref[rid] = cache[key]
     pos = {r: 0 for r in reqs}
-    worst = 0.0
+    worst, over, count = 0.0, 0, 0
     for s in steps:
         row = 0
         for e in s["entries"]:
@@ -120,9 +120,15 @@ def check_logits(model_dir: str, reqs: Dict[str, List[int]], steps: List[dict], 
                 assert np.isfinite(gl).all(), f"step {s['step']} request {e['id']} position {p}: logits are not finite"
                 diff = gl - r
                 err = float(np.sqrt(np.mean((diff - diff.mean()) ** 2)) / max(np.sqrt(np.mean((r - r.mean()) ** 2)), 1e-30))
-                assert err < TOL[dtype], (f"step {s['step']} request {e['id']} position {p} "
-                                          f"(portion starts at {pos[e['id']]}): error {err:.3e} > {TOL[dtype]:.0e}")
+                # float32: every position within the tolerance.  bfloat16: a position whose logits lie close together
+                # magnifies the rounding it has inherited, so one position in fifty (or one) may be up to half again over
+                hard = TOL[dtype] * (1.5 if dtype == "bfloat16" else 1.0)
+                assert err < hard, (f"step {s['step']} request {e['id']} position {p} "
+                                    f"(portion starts at {pos[e['id']]}): error {err:.3e} > {hard:.1e}")
+                over += err >= TOL[dtype]
+                count += 1
                 worst = max(worst, err)
                 row += 1
             pos[e["id"]] += len(e["tokens"])
+    assert over <= max(1, count // 50), f"{over} of {count} positions are over {TOL[dtype]:.0e} (worst {worst:.3e})"
     return worst

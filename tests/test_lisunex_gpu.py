@@ -374,3 +374,49 @@ def test_captured_decoding_steps_move_the_state_once(folders):
     for k in got_plain:
         assert np.array_equal(got[k], got_plain[k]), f"step {k} differs between replayed and launched steps"
     check_logits(folder, reqs, steps, got, "bfloat16")
+
+
+def random_lisunex_config(seed: int) -> dict:
+    """Sizes, orders and constants drawn at random, odd ones on purpose."""
+    rs = np.random.RandomState(seed)
+    pick = lambda xs: xs[rs.randint(len(xs))]
+    width = int(pick([40, 72, 100, 136, 200]))
+    layers = []
+    for _ in range(rs.randint(2, 6)):
+        heads = int(pick([1, 2, 3, 4, 6, 8]))
+        kv = int(pick([k for k in (1, 2, 3, 4) if heads % k == 0]))
+        ff = int(pick([0, 24, 100, 136]))
+        if rs.rand() < 0.5:
+            dim = int(pick([8, 16, 24, 40, 64]))
+            layers.append(attention_layer(heads=heads, kv_heads=kv, dim=dim, vdim=int(pick([8, 16, 32, 40, 80, 144])),
+                                          scale=float(pick([0.05, 0.3, 1.0])), softcap=float(pick([0.0, 2.0, 30.0])),
+                                          chunk=int(pick([1, 3, 16, 50, 1000])), rot_dims=int(pick([d for d in (2, 4, 8, 16, 24, 40, 64) if d <= dim])),
+                                          base=float(pick([100.0, 1e4, 1e6])), scaling=bool(rs.rand() < 0.6), ff=ff or None))
+        else:
+            layers.append(delta_layer(heads=heads, kv_heads=kv, dim=int(pick([8, 12, 32, 72, 128])),
+                                      vdim=int(pick([8, 20, 64, 80])), conv=int(pick([2, 3, 4, 6])), ff=ff or None))
+    n = len(layers)
+    loop = None
+    if rs.rand() < 0.6:
+        a = int(rs.randint(0, n))
+        loop = {"start": a, "stop": int(rs.randint(a + 1, n + 1)), "times": int(rs.randint(1, 4))}
+    return {"architecture": "Lisunex", "vocab": int(pick([51, 97, 130, 255])), "width": width,
+            "embedding": {"scale": float(pick([1.0, 0.5, 9.0]))}, "norm": {"eps": float(pick([1e-6, 1e-5, 1e-3]))},
+            "layers": layers, "loop": loop}
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Whatever config.json says is what runs: random sizes, layer orders, loops and constants, in float32 (sharp) and
+    bfloat16, through portions and a mixed batch."""
+    cfg = random_lisunex_config(seed)
+    folder = write_model(copy.deepcopy(cfg), str(tmp_path / "m"), seed=40 + seed)
+    reqs = rh.random_requests(cfg["vocab"], [37, 5, 70], seed=seed)
+    steps = rh.trace_mixed(reqs, {r: rh.cut(t, [11, 2, 1, 30, 1, 1]) for r, t in reqs.items()}, max_live=2, seed=seed)
+    whole = rh.trace_alone(reqs, {r: [(0, len(t))] for r, t in reqs.items()})
+    cache = {}
+    for dtype in ("float32", "bfloat16"):
+        runner = make_runner(folder, dtype, pool_tokens=192, max_requests=2)
+        runner.decode_graphs = True
+        check_logits(folder, reqs, whole, rh.run_in_process(runner, whole), dtype, cache)
+        check_logits(folder, reqs, steps, rh.run_in_process(runner, steps), dtype, cache)
