@@ -229,17 +229,12 @@ def test_gated_delta_part(dtype, nh, kvh, d, dv, taps):
                                                       conv_taps=taps, norm_eps=1e-5)), rt=rt, width=width, prefix="m.", shared={})
     w = weights_for(mixer, 7, 0.25)
     w["m.A_log"] = torch.log(torch.linspace(0.02, 1.5, nh)).to(torch.bfloat16).float()
-    if taps == 1:
-        w = {k: v for k, v in w.items() if "conv" not in k}
     mixer.load(w.__getitem__, rt)
     runner = ModelRunner(OneMixer(mixer), rt, 16, 256, 3, 256)
     assert runner.storage.state[0].shape == (3 + 1, (taps - 1) * (2 * kvh * d + nh * dv) + nh * d * dv)
     x = (torch.randn(t, width, generator=torch.Generator().manual_seed(8)) * 0.8).to(dtype)
     wd = {k[2:].replace("_proj.weight", "").replace("_conv.weight", ".conv").replace("norm.weight", "norm"): v.double()
           for k, v in w.items()}
-    if taps == 1:
-        for k, rows in (("q", kvh * d), ("k", kvh * d), ("v", nh * dv)):
-            wd[k + ".conv"] = torch.ones(rows, 1, dtype=torch.float64)
     ref = pl.delta_mixer(x.double(), wd, "", dict(heads=nh, kv_heads=kvh, dim=d, vdim=dv), 1e-5)
     whole = step_part(runner, mixer, x, [(0, t)])
     assert rel(whole, ref) < PART_TOL[dtype]

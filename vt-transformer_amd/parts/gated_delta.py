@@ -38,7 +38,7 @@ class GatedDeltaMixer(Part):
                  value_dim: int, conv_taps: int, norm_eps: float, shared: Optional[dict] = None,
                  names: Optional[Dict[str, str]] = None):
         """num_heads value heads of value_dim, num_kv_heads query/key heads of key_dim (value head h reads query/key
-        head h // (num_heads / num_kv_heads)); conv_taps: length of the convolutions (1: none); norm_eps: eps of
+        head h // (num_heads / num_kv_heads)); conv_taps: length of the convolutions (1: a factor per channel); norm_eps: eps of
         the output's norm; names: tensor names behind the prefix for q, k, v, g, o (matrices), q_conv, k_conv, v_conv
         ([channels, taps], the last column is the current token's), b and a (write strength and decay, one row per
         head), A_log, dt_bias (per head) and norm (per value channel)."""
@@ -85,10 +85,10 @@ class GatedDeltaMixer(Part):
             nm["dt_bias"]: TensorDecl((self.nh,), "bias"),
             nm["norm"]: TensorDecl((self.dv,), "gain"),
         }
-        if self.taps > 1:
-            t[nm["q_conv"]] = TensorDecl((kd, self.taps), "bias")
-            t[nm["k_conv"]] = TensorDecl((kd, self.taps), "bias")
-            t[nm["v_conv"]] = TensorDecl((vd, self.taps), "bias")
+        # (with one tap the "convolution" is a factor per channel: the tensors are there all the same)
+        t[nm["q_conv"]] = TensorDecl((kd, self.taps), "bias")
+        t[nm["k_conv"]] = TensorDecl((kd, self.taps), "bias")
+        t[nm["v_conv"]] = TensorDecl((vd, self.taps), "bias")
         return t
 
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
@@ -99,10 +99,7 @@ class GatedDeltaMixer(Part):
         self.w_o = rt.place(get(nm["o"]), "matrix")
         self.p_in, self.p_o = rt.pack(self.w_in), rt.pack(self.w_o)
         self.w_in, self.w_o = rt.row_major(self.w_in, self.p_in), rt.row_major(self.w_o, self.p_o)
-        if self.taps > 1:
-            self.conv_w = torch.cat([rt.place(get(nm[k]), "bias") for k in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
-        else:
-            self.conv_w = torch.ones((self.channels, 1), dtype=torch.float32, device=rt.device)
+        self.conv_w = torch.cat([rt.place(get(nm[k]), "bias") for k in ("q_conv", "k_conv", "v_conv")], dim=0).contiguous()
         self.a_log, self.dt_bias = rt.place(get(nm["A_log"]), "bias"), rt.place(get(nm["dt_bias"]), "bias")
         self.norm_w = rt.place(get(nm["norm"]), "gain")
 
