@@ -13,6 +13,12 @@
 //                   score = cap * tanh(scale * q.k / cap) (cap 0: none); key j is seen from position i if j <= i,
 //                   i - j < window (window 0: no bound) and j >= floor(i / chunk) * chunk (chunk 0: no bound);
 //                   out = softmax(score) V * sigmoid(gate[token][head]) (no gate pointer: no gate).
+//                   With `slopes`, slopes[head] * (i - j) is taken off the score of key j (behind the cap); with
+//                   `sink`, exp(sink[head]) joins the softmax's denominator and nothing else: a key that holds no
+//                   value.
+//   vt_qk_prepare also scales the queries of position p by 1 + coef * ln(floor((p + 1) / every) + 1) (every 0: not),
+//                   and mixes values across layers: vmix 1 leaves the token's values in `v_first` (float32), vmix 2
+//                   writes (1 - lambda) v + lambda v_first into the pages instead of v.
 #include "vt_common.h"
 #include <math.h>
 
@@ -32,6 +38,11 @@ struct PrepArgs {
     long long ldx;
     int H, G, D, Dv, rot, max_pos, page_size, max_blocks, num_pages, write_kv, unit_rms;
     float eps;
+    float q_temp_coef;      // queries times 1 + coef * ln(floor((pos + 1) / every) + 1); every 0: no factor
+    int q_temp_every;
+    int vmix;               // 0: none; 1: the values go to v_first as well; 2: the pages get (1 - lambda) v + lambda v_first
+    float* v_first;         // [n][G * Dv] float32
+    const float* v_lambda;  // one float on the device
 };
 
 template <typename TI, typename TC>
@@ -83,6 +94,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(PrepArgs a) {
                 ss = wave_sum(ss);
                 r = 1.0f / sqrtf(ss / (float)a.D + a.eps);
             }
+            if (is_q && a.q_temp_every > 0) r *= 1.0f + a.q_temp_coef * logf((float)((pos + 1) / a.q_temp_every) + 1.0f);
             if (is_q) {
                 TC* dst = (TC*)a.q_out + ((size_t)t * a.H + u) * a.D;
 #pragma unroll
@@ -104,7 +116,14 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(PrepArgs a) {
             const int g = u - a.H - a.G;
             const TI* src = x + (size_t)(a.H + a.G) * a.D + (size_t)g * a.Dv;
             TC* dst = (TC*)a.v_pages + ((size_t)page_no * a.G + g) * a.Dv * a.page_size + page_slot;
-            for (int d = lane; d < a.Dv; d += 64) store_f32<TC>(dst, (size_t)d * a.page_size, load_f32<TI>(src, d));
+            float* vf = a.v_first + ((size_t)t * a.G + g) * a.Dv;
+            const float lam = a.vmix == 2 ? a.v_lambda[0] : 0.f;
+            for (int d = lane; d < a.Dv; d += 64) {
+                float v = load_f32<TI>(src, d);
+                if (a.vmix == 1) vf[d] = v;
+                else if (a.vmix == 2) v = (1.0f - lam) * v + lam * vf[d];
+                store_f32<TC>(dst, (size_t)d * a.page_size, v);
+            }
         }
     }
 }
@@ -113,6 +132,7 @@ extern "C" int vt_qk_prepare(const void* x, int x_dtype, long long ldx, const fl
                              int max_pos, const int* positions, const int* tok_entry, const int* block_table,
                              int max_blocks, void* q_out, void* k_pages, void* v_pages, int cache_dtype, int page_size,
                              int num_pages, int n, int H, int G, int D, int Dv, int write_kv, int unit_rms, float eps,
+                             float q_temp_coef, int q_temp_every, int vmix, float* v_first, const float* v_lambda,
                              hipStream_t stream) {
     VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_qk_prepare: bad heads %d/%d", H, G);
     VT_REQUIRE(D > 0 && D <= 256 && Dv > 0, "vt_qk_prepare: head sizes %d/%d (keys up to 256)", D, Dv);
@@ -122,12 +142,16 @@ extern "C" int vt_qk_prepare(const void* x, int x_dtype, long long ldx, const fl
                "vt_qk_prepare: rows of %lld elements are too short", ldx);
     VT_REQUIRE(!write_kv || (page_size > 0 && max_blocks > 0 && num_pages > 0 && block_table && k_pages && v_pages),
                "vt_qk_prepare: bad cache sizes");
+    VT_REQUIRE(q_temp_every >= 0, "vt_qk_prepare: a query factor every %d positions", q_temp_every);
+    VT_REQUIRE(vmix == 0 || ((vmix == 1 || vmix == 2) && write_kv && v_first && (vmix == 1 || v_lambda)),
+               "vt_qk_prepare: value mixing %d without its buffers", vmix);
     if (n == 0) return 0;
     PrepArgs a;
     a.x = x; a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.tok_entry = tok_entry; a.block_table = block_table;
     a.q_out = q_out; a.k_pages = k_pages; a.v_pages = v_pages; a.ldx = ldx; a.H = H; a.G = G; a.D = D; a.Dv = Dv; a.rot = rot;
     a.max_pos = max_pos; a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages; a.write_kv = write_kv;
-    a.unit_rms = unit_rms; a.eps = eps;
+    a.unit_rms = unit_rms; a.eps = eps; a.q_temp_coef = q_temp_coef; a.q_temp_every = q_temp_every; a.vmix = vmix;
+    a.v_first = v_first; a.v_lambda = v_lambda;
     // few tokens: a wave per head, over several blocks per token; many tokens: a block per token goes through its heads
     const int units = H + (write_kv ? 2 * G : 0);
     const dim3 grid(n, n >= 1024 ? 1 : (units + 3) / 4);
@@ -148,6 +172,8 @@ struct MaskedArgs {
     const int* tok_entry;
     const int* block_table;
     const void* gate;       // gate[t * ldg + h], or null
+    const float* sink;      // [H], or null: exp(sink[h]) joins the denominator
+    const float* slopes;    // [H], or null: slopes[h] * (position - key index) is taken off every score
     void* out;              // [n][H][Dv]
     long long ldg;
     int H, G, D, Dv, page_size, max_blocks, num_pages, window, chunk;
@@ -173,6 +199,7 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
     if (a.window > 0) lo = max(lo, pos - a.window + 1);
     const TC* kp = (const TC*)a.k_pages;
     const TC* vp = (const TC*)a.v_pages;
+    const float slope = a.slopes ? a.slopes[h] : 0.f;
 
     for (int d = tid; d < D; d += KEYS) qs[d] = load_f32<TC>((const TC*)a.q, ((size_t)t * a.H + h) * D + d);
     __syncthreads();
@@ -195,6 +222,7 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
                 for (int d = 0; d < D; ++d) dot = fmaf(qs[d], load_f32<TC>(kr, d), dot);
                 s = dot * a.scale;
                 if (a.cap > 0.f) s = a.cap * tanhf(s / a.cap);
+                if (a.slopes) s -= slope * (float)(pos - j);
             } else {
                 s = __int_as_float(0x7fc00000);  // a missing page must show, not pass as a masked key
             }
@@ -228,6 +256,14 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
         __syncthreads();
         m = m_new;
     }
+    if (a.sink) {
+        // the sink is one more score with no value behind it
+        const float sk = a.sink[h];
+        const float m_all = fmaxf(m, sk);
+        const float keep = expf(m - m_all);
+        l = l * keep + expf(sk - m_all);
+        acc *= keep;
+    }
     if (tid < Dv) {
         float o = acc / l;
         if (a.gate) {
@@ -242,7 +278,7 @@ extern "C" int vt_attn_masked(const void* q, const void* k_pages, const void* v_
                               const int* tok_entry, const int* block_table, const void* gate, int gate_dtype,
                               long long ldg, void* out, int n, int H, int G, int D, int Dv, int page_size,
                               int max_blocks, int num_pages, int window, int chunk, float scale, float cap,
-                              hipStream_t stream) {
+                              const float* sink, const float* slopes, hipStream_t stream) {
     VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked: bad heads %d/%d", H, G);
     VT_REQUIRE(D > 0 && Dv > 0 && Dv <= 256, "vt_attn_masked: head sizes %d/%d (values up to 256)", D, Dv);
     VT_REQUIRE(page_size > 0 && max_blocks > 0 && num_pages > 0, "vt_attn_masked: bad cache sizes");
@@ -253,7 +289,7 @@ extern "C" int vt_attn_masked(const void* q, const void* k_pages, const void* v_
     a.q = q; a.k_pages = k_pages; a.v_pages = v_pages; a.positions = positions; a.tok_entry = tok_entry;
     a.block_table = block_table; a.gate = gate; a.out = out; a.ldg = ldg; a.H = H; a.G = G; a.D = D; a.Dv = Dv;
     a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages; a.window = window; a.chunk = chunk;
-    a.scale = scale; a.cap = cap;
+    a.scale = scale; a.cap = cap; a.sink = sink; a.slopes = slopes;
     const size_t shmem = (size_t)(D + 2 * KEYS) * sizeof(float);
     const dim3 grid(n, H);
     if (dtype == VT_F32) {

@@ -11,6 +11,8 @@
 //     O^T += V^T P^T   [Dv x 16 queries]; A = V^T from the page ([kv head][Dv][slot]: a lane reads 4 consecutive keys of
 //                      its value element), B = P^T, which is exactly what the lane holds of S^T
 // so the probabilities never leave the registers.  Scores, softmax and sums are float32.
+// With `slopes`, slopes[head] * (position - key index) is taken off every score; with `sink`, exp(sink[head]) joins
+// the softmax's denominator (a key that holds no value).
 #include "vt_common.h"
 #include <math.h>
 
@@ -33,6 +35,8 @@ struct MfmaArgs {
     const int* block_table;
     const int* tiles;       // [n_tiles][2]: first row, rows (1..16), all of one request
     const void* gate;       // gate[t * ldg + h], or null
+    const float* sink;      // [H] or null
+    const float* slopes;    // [H] or null
     bf16_t* out;            // [n][H][Dv]
     long long ldg;
     int n_tiles, H, G, page_size, max_blocks, num_pages, window, chunk, gate_f32;
@@ -82,6 +86,7 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
     const float LOG2E = 1.4426950408889634f;
     const float c1 = a.cap > 0.f ? a.scale * 2.0f * LOG2E / a.cap : a.scale * LOG2E;
     const float c2 = a.cap * LOG2E;
+    const float slope2 = a.slopes ? a.slopes[h] * LOG2E : 0.f;
     const int lo_last = [&] {
         int v = a.chunk > 0 ? (pos_last / a.chunk) * a.chunk : 0;
         if (a.window > 0) v = max(v, pos_last - a.window + 1);
@@ -143,6 +148,10 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
                 sc[i] = x;
             }
         }
+        if (a.slopes) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sc[i] -= slope2 * (float)(pos - (kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3)));
+        }
         // a turn that every row sees whole needs no mask
         const bool whole = kt + 31 <= pos_first && kt >= lo_last && ok_now[0] && ok_now[1];
         if (!whole) {
@@ -181,6 +190,15 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_kernel(MfmaArgs a) {
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (!row_ok) return;
+    if (a.sink) {
+        // the sink is one more score with no value behind it (scores are kept times log2 e)
+        const float sk = a.sink[h] * LOG2E;
+        const float m_all = fmaxf(m, sk);
+        const float keep = __builtin_amdgcn_exp2f(m - m_all);
+        l = l * keep + __builtin_amdgcn_exp2f(sk - m_all);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[v] *= keep;
+    }
     float gate = 1.f;
     if (a.gate) {
         const size_t gi = (size_t)t * a.ldg + h;
@@ -253,6 +271,7 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
     const float LOG2E = 1.4426950408889634f;
     const float c1 = a.cap > 0.f ? a.scale * 2.0f * LOG2E / a.cap : a.scale * LOG2E;
     const float c2 = a.cap * LOG2E;
+    const float slope2 = a.slopes ? a.slopes[h] * LOG2E : 0.f;
 
     auto page_of = [&](int kt) -> int {
         const int blk = kt / ps;
@@ -345,6 +364,10 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
                 sc[i] = x;
             }
         }
+        if (a.slopes) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) sc[i] -= slope2 * (float)(pos - (kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3)));
+        }
         const bool whole = kt + 31 <= pos_first && kt >= lo_last && ok_now[0] && ok_now[1];
         if (!whole) {
 #pragma unroll
@@ -386,6 +409,15 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (!row_ok) return;
+    if (a.sink) {
+        // the sink is one more score with no value behind it (scores are kept times log2 e)
+        const float sk = a.sink[h] * LOG2E;
+        const float m_all = fmaxf(m, sk);
+        const float keep = __builtin_amdgcn_exp2f(m - m_all);
+        l = l * keep + __builtin_amdgcn_exp2f(sk - m_all);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[v] *= keep;
+    }
     float gate = 1.f;
     if (a.gate) {
         const size_t gi = (size_t)t * a.ldg + h;
@@ -411,7 +443,7 @@ extern "C" int vt_attn_masked_mfma(const void* q, const void* k_pages, const voi
                                    const int* tok_entry, const int* block_table, const int* tiles, int n_tiles,
                                    const void* gate, int gate_dtype, long long ldg, void* out, int H, int G, int D, int Dv,
                                    int page_size, int max_blocks, int num_pages, int window, int chunk, float scale,
-                                   float cap, hipStream_t stream) {
+                                   float cap, const float* sink, const float* slopes, hipStream_t stream) {
     VT_REQUIRE(D == VT_KEY_DIM && Dv == VT_VALUE_DIM, "vt_attn_masked_mfma: built for heads of %d/%d, called with %d/%d",
                VT_KEY_DIM, VT_VALUE_DIM, D, Dv);
     VT_REQUIRE(n_tiles >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked_mfma: bad heads %d/%d", H, G);
@@ -425,6 +457,7 @@ extern "C" int vt_attn_masked_mfma(const void* q, const void* k_pages, const voi
     a.tok_entry = tok_entry; a.block_table = block_table; a.tiles = tiles; a.gate = gate; a.out = (bf16_t*)out; a.ldg = ldg;
     a.n_tiles = n_tiles; a.H = H; a.G = G; a.page_size = page_size; a.max_blocks = max_blocks; a.num_pages = num_pages;
     a.window = window; a.chunk = chunk; a.gate_f32 = gate_dtype == VT_F32; a.scale = scale; a.cap = cap;
+    a.sink = sink; a.slopes = slopes;
     const long long items = (long long)n_tiles * H;
     if ((H / G) % 4 == 0)       // four heads of one key/value group to a block: they share what they read
         attn_masked_mfma_shared_kernel<<<(unsigned)(items / 4), 256, 0, stream>>>(a);

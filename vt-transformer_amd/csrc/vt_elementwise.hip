@@ -347,6 +347,81 @@ extern "C" int vt_silu_mul(const void* gu, int in_dtype, void* out, int out_dtyp
 }
 
 // ---------------------------------------------------------------------------
+// A gated unit with bounds: g = min(gu[t, i], limit), u = clamp(gu[t, inter + i], -limit, limit),
+// out[t, i] = g * sigmoid(alpha * g) * (u + shift).  limit <= 0: no bounds.  (alpha 1, shift 0 and no bounds is
+// vt_silu_mul.)  A thread takes four columns where the width is a multiple of 4.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ float bounded_gate(float g, float u, float alpha, float limit, float shift) {
+    if (limit > 0.f) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+    }
+    return g / (1.f + expf(-alpha * g)) * (u + shift);
+}
+template <typename TI, typename TO>
+__global__ void gated_act_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter, float alpha, float limit,
+                                 float shift) {
+    int t = blockIdx.y;
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= inter) return;
+    const TI* row = gu + (size_t)t * 2 * inter;
+    store_f32<TO>(out + (size_t)t * inter, i, bounded_gate(load_f32<TI>(row, i), load_f32<TI>(row, (size_t)inter + i), alpha, limit, shift));
+}
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void gated_act_vec_kernel(const TI* __restrict__ gu, TO* __restrict__ out, int inter,
+                                                           int n, float alpha, float limit, float shift) {
+    const int qpr = inter >> 2;
+    const long long total = (long long)qpr * n;
+    for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256) {
+        const long long t = idx / qpr;
+        const int i = (int)(idx - t * qpr) * 4;
+        const TI* row = gu + (size_t)t * 2 * inter;
+        const float4 g = load4(row + i), u = load4(row + inter + i);
+        store4(out + (size_t)t * inter + i,
+               make_float4(bounded_gate(g.x, u.x, alpha, limit, shift), bounded_gate(g.y, u.y, alpha, limit, shift),
+                           bounded_gate(g.z, u.z, alpha, limit, shift), bounded_gate(g.w, u.w, alpha, limit, shift)));
+    }
+}
+template <typename TI, typename TO>
+static void launch_gated_act(const void* gu, void* out, int n, int inter, float alpha, float limit, float shift,
+                             hipStream_t stream) {
+    if (inter % 4 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
+        long long blocks = ((long long)(inter / 4) * n + 255) / 256;
+        if (blocks > 16384) blocks = 16384;
+        gated_act_vec_kernel<TI, TO><<<(unsigned)blocks, 256, 0, stream>>>((const TI*)gu, (TO*)out, inter, n, alpha, limit, shift);
+    } else {
+        gated_act_kernel<TI, TO><<<dim3((inter + 255) / 256, n), 256, 0, stream>>>((const TI*)gu, (TO*)out, inter, alpha, limit, shift);
+    }
+}
+extern "C" int vt_gated_act(const void* gu, int in_dtype, void* out, int out_dtype, int n, int inter, float alpha,
+                            float limit, float shift, hipStream_t stream) {
+    VT_REQUIRE(n >= 0 && inter > 0, "vt_gated_act: bad sizes n=%d inter=%d", n, inter);
+    if (n == 0) return 0;
+    VT_REQUIRE(n <= 65535, "vt_gated_act: more than 65535 rows (%d)", n);
+    if (in_dtype == VT_F32 && out_dtype == VT_F32) launch_gated_act<float, float>(gu, out, n, inter, alpha, limit, shift, stream);
+    else if (in_dtype == VT_F32 && out_dtype == VT_BF16) launch_gated_act<float, bf16_t>(gu, out, n, inter, alpha, limit, shift, stream);
+    else if (in_dtype == VT_BF16 && out_dtype == VT_BF16) launch_gated_act<bf16_t, bf16_t>(gu, out, n, inter, alpha, limit, shift, stream);
+    else return vt_fail("vt_gated_act: unknown dtypes %d -> %d", in_dtype, out_dtype);
+    VT_CHECK_LAUNCH("vt_gated_act");
+    return 0;
+}
+
+// x <- cap * tanh(x / cap), in place (logits bounded to (-cap, cap))
+__global__ void tanh_cap_kernel(float* __restrict__ x, long long n, float cap) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+        x[i] = cap * tanhf(x[i] / cap);
+}
+extern "C" int vt_tanh_cap(float* x, long long n, float cap, hipStream_t stream) {
+    VT_REQUIRE(n >= 0 && cap > 0.f, "vt_tanh_cap: bad arguments");
+    if (n == 0) return 0;
+    long long blocks = (n + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    tanh_cap_kernel<<<(unsigned)blocks, 256, 0, stream>>>(x, n, cap);
+    VT_CHECK_LAUNCH("vt_tanh_cap");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
 // Rotary encoding of queries and keys and the write of keys and values into
 // cache pages, one block per (token, head).
 //

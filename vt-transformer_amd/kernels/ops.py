@@ -158,6 +158,30 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def gated_act(gu: torch.Tensor, out: torch.Tensor, alpha: float = 1.0, limit: float = 0.0, shift: float = 0.0) -> torch.Tensor:
+    """gu [n, 2 I] (gate columns, then up columns) -> out [n, I] = g sigmoid(alpha g) (u + shift) with g = min(gate,
+    limit) and u = clamp(up, -limit, limit); limit 0: no bounds."""
+    n, two_i = gu.shape
+    _chk(gu, "gated_act.gu")
+    _chk(out, "gated_act.out", None, (n, two_i // 2))
+    if two_i % 2:
+        raise KernelError(f"gated_act: input width {two_i} is odd")
+    if out.dtype == torch.float32 and gu.dtype != torch.float32:
+        raise KernelError("gated_act: float32 results need float32 inputs")
+    _run(load_lib("vt_elementwise", half=_half(gu, out)), "vt_gated_act", _ptr(gu), _i(_code(gu)), _ptr(out), _i(_code(out)),
+         _i(n), _i(two_i // 2), _f(alpha), _f(limit), _f(shift), _stream())
+    return out
+
+
+def tanh_cap(x: torch.Tensor, cap: float) -> torch.Tensor:
+    """x <- cap * tanh(x / cap), in place; float32."""
+    _chk(x, "tanh_cap.x", torch.float32)
+    if not cap > 0:
+        raise KernelError(f"tanh_cap: cap {cap} must be positive")
+    _run(_any_build("vt_elementwise"), "vt_tanh_cap", _ptr(x), ctypes.c_longlong(x.numel()), _f(cap), _stream())
+    return x
+
+
 def gather_rows(x: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
     _chk(x, "gather_rows.x")
     n = rows.numel() if rows is not None else x.shape[0]
@@ -664,11 +688,16 @@ MASKED_MAX_VALUE_DIM = 256
 def qk_prepare(x: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
                tok_entry: torch.Tensor, block_table: Optional[torch.Tensor], q_out: torch.Tensor,
                k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], n_heads: int, n_kv: int, key_dim: int,
-               value_dim: int, unit_rms_eps: Optional[float], write_kv: bool = True) -> None:
+               value_dim: int, unit_rms_eps: Optional[float], write_kv: bool = True,
+               q_temp: Optional[tuple] = None, v_first: Optional[torch.Tensor] = None,
+               v_lambda: Optional[torch.Tensor] = None) -> None:
     """x [n, >= (H + G) D + G Dv]: query heads, key heads, value heads.  Rotates the leading 2 * cos.shape[1] elements
     of every query and key head by the tables' angles at `positions`, divides each head by its root mean square
     (eps inside the root) unless unit_rms_eps is None, writes queries to q_out [n, H * D] and, with write_kv, keys and
-    values into their pages ([page][kv][slot][D] and, transposed, [page][kv][Dv][slot])."""
+    values into their pages ([page][kv][slot][D] and, transposed, [page][kv][Dv][slot]).
+    q_temp (coef, every): the queries of position p times 1 + coef ln(floor((p + 1) / every) + 1).
+    v_first (float32 [n, G * Dv]): without v_lambda the tokens' values are left there as well; with v_lambda (one
+    float32 on the device) the pages get (1 - lambda) v + lambda v_first instead of v."""
     n = x.shape[0]
     _chk(x, "qk_prepare.x")
     need = (n_heads + (n_kv if write_kv else 0)) * key_dim + (n_kv * value_dim if write_kv else 0)
@@ -698,20 +727,38 @@ def qk_prepare(x: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch
         _chk(v_pages, "qk_prepare.v_pages", q_out.dtype, (num_pages, n_kv, value_dim, page_size))
         _chk(block_table, "qk_prepare.block_table", torch.int32)
         max_blocks = block_table.shape[1]
+    coef, every = (float(q_temp[0]), int(q_temp[1])) if q_temp else (0.0, 0)
+    if q_temp and every <= 0:
+        raise KernelError(f"qk_prepare: a query factor every {every} positions")
+    vmix = 0
+    if v_first is not None:
+        if not write_kv:
+            raise KernelError("qk_prepare: values are mixed on their way into the pages")
+        _chk(v_first, "qk_prepare.v_first", torch.float32, (n, n_kv * value_dim))
+        vmix = 1
+        if v_lambda is not None:
+            _chk(v_lambda, "qk_prepare.v_lambda", torch.float32)
+            if v_lambda.numel() != 1:
+                raise KernelError("qk_prepare.v_lambda: one number")
+            vmix = 2
     _run(load_lib("vt_attn_masked", half=_half(x, q_out)), "vt_qk_prepare", _ptr(x), _i(_code(x)),
          ctypes.c_longlong(x.stride(0)), _ptr(cos), _ptr(sin), _i(rot), _i(max_pos), _ptr(positions), _ptr(tok_entry),
          _ptr(block_table), _i(max_blocks), _ptr(q_out), _ptr(k_pages), _ptr(v_pages), _i(_code(q_out)), _i(page_size),
          _i(num_pages), _i(n), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(1 if write_kv else 0),
-         _i(0 if unit_rms_eps is None else 1), _f(unit_rms_eps or 0.0), _stream())
+         _i(0 if unit_rms_eps is None else 1), _f(unit_rms_eps or 0.0), _f(coef), _i(every), _i(vmix), _ptr(v_first),
+         _ptr(v_lambda if vmix == 2 else None), _stream())
 
 
 def attention_masked(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, positions: torch.Tensor,
                      tok_entry: torch.Tensor, block_table: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int,
                      key_dim: int, value_dim: int, scale: float, cap: float = 0.0, window: int = 0, chunk: int = 0,
-                     gate: Optional[torch.Tensor] = None, gate_column: int = 0) -> torch.Tensor:
+                     gate: Optional[torch.Tensor] = None, gate_column: int = 0, sink: Optional[torch.Tensor] = None,
+                     slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out [n, H * Dv] = softmax over the seen keys of cap * tanh(scale q.k / cap) (cap 0: scale q.k), times V, times
     sigmoid(gate[:, gate_column + head]) if `gate` (a 2-d tensor whose rows are the tokens') is given.  Key j is seen
-    from position i if j <= i, i - j < window (0: unbounded) and j is in i's chunk of `chunk` positions (0: unbounded)."""
+    from position i if j <= i, i - j < window (0: unbounded) and j is in i's chunk of `chunk` positions (0: unbounded).
+    slopes (float32 [H]): slopes[h] * (i - j) is taken off the score; sink (float32 [H]): exp(sink[h]) is added to the
+    softmax's denominator."""
     n = q.shape[0]
     num_pages, kvh, page_size, d = k_pages.shape
     dt = q.dtype
@@ -733,11 +780,18 @@ def attention_masked(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
             raise KernelError("attention_masked: float32 attention takes float32 gates")
         gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
         gcode, ldg = _code(gate), gate.stride(0)
+    _per_head(sink, "attention_masked.sink", n_heads)
+    _per_head(slopes, "attention_masked.slopes", n_heads)
     _run(load_lib("vt_attn_masked", half=_half(q, gate)), "vt_attn_masked", _ptr(q), _ptr(k_pages), _ptr(v_pages), _i(_code(q)),
          _ptr(positions), _ptr(tok_entry), _ptr(block_table), gptr, _i(gcode), ctypes.c_longlong(ldg), _ptr(out), _i(n),
          _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size), _i(block_table.shape[1]), _i(num_pages),
-         _i(window), _i(chunk), _f(scale), _f(cap), _stream())
+         _i(window), _i(chunk), _f(scale), _f(cap), _ptr(sink), _ptr(slopes), _stream())
     return out
+
+
+def _per_head(t: Optional[torch.Tensor], name: str, n_heads: int) -> None:
+    if t is not None:
+        _chk(t, name, torch.float32, (n_heads,))
 
 
 def attention_masked_mfma_takes(key_dim: int, value_dim: int, page_size: int) -> bool:
@@ -750,7 +804,8 @@ def attention_masked_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
                           tok_entry: torch.Tensor, block_table: torch.Tensor, tiles: torch.Tensor, out: torch.Tensor,
                           n_heads: int, n_kv: int, key_dim: int, value_dim: int, scale: float, cap: float = 0.0,
                           window: int = 0, chunk: int = 0, gate: Optional[torch.Tensor] = None,
-                          gate_column: int = 0) -> torch.Tensor:
+                          gate_column: int = 0, sink: Optional[torch.Tensor] = None,
+                          slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
     """attention_masked for the 16-bit types on the matrix cores.  tiles: int32 [n_tiles, 2], (first row, rows) of
     runs of up to 16 consecutive tokens of one request that together cover every token of the step once."""
     n = q.shape[0]
@@ -776,11 +831,102 @@ def attention_masked_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
             raise KernelError(f"attention_masked_mfma.gate: shape {tuple(gate.shape)} has no {n_heads} columns from {gate_column}")
         gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
         gcode, ldg = _code(gate), gate.stride(0)
+    _per_head(sink, "attention_masked_mfma.sink", n_heads)
+    _per_head(slopes, "attention_masked_mfma.slopes", n_heads)
     _run(load_lib("vt_attn_masked_mfma", (key_dim, value_dim), half=_half(q, gate)), "vt_attn_masked_mfma", _ptr(q), _ptr(k_pages),
          _ptr(v_pages), _ptr(positions), _ptr(tok_entry), _ptr(block_table), _ptr(tiles), _i(tiles.numel() // 2), gptr,
          _i(gcode), ctypes.c_longlong(ldg), _ptr(out), _i(n_heads), _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size),
-         _i(block_table.shape[1]), _i(num_pages), _i(window), _i(chunk), _f(scale), _f(cap), _stream())
+         _i(block_table.shape[1]), _i(num_pages), _i(window), _i(chunk), _f(scale), _f(cap), _ptr(sink), _ptr(slopes),
+         _stream())
     return out
+
+
+# ---------------------------------------------------------------------------
+# attention over a low-rank cache (vt_latent.hip): what stands around the masked attention kernels
+HEAD_LINEAR_MAX_IN = 8192
+
+
+def latent_prepare(x: torch.Tensor, q_column: int, c_column: int, norm_w: torch.Tensor, eps: float,
+                   cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
+                   tok_entry: torch.Tensor, block_table: torch.Tensor, q_out: torch.Tensor, k_pages: torch.Tensor,
+                   v_pages: torch.Tensor, n_heads: int, plain_dim: int, rot_dim: int, rank: int) -> None:
+    """x [n, ...]: from column q_column the heads' queries, each [plain_dim | rot_dim]; from column c_column the
+    low-rank part [rank | rot_dim].  c = the first `rank` over their root mean square (eps inside the root) times
+    norm_w goes into the key page's leading `rank` elements and, transposed, into the value page; the `rot_dim`
+    behind it, its leading 2 * cos.shape[1] elements rotated by the tables' angles at `positions`, into the key page
+    behind c; every head's rot_dim query elements, rotated alike, into q_out[:, head, rank:].
+    q_out [n, H * (rank + rot_dim)], k_pages [pages, 1, page_size, rank + rot_dim], v_pages [pages, 1, rank, page_size]."""
+    n = x.shape[0]
+    dk = rank + rot_dim
+    _chk(x, "latent_prepare.x")
+    if x.dim() != 2 or x.shape[1] < max(q_column + n_heads * (plain_dim + rot_dim), c_column + dk) or min(q_column, c_column) < 0:
+        raise KernelError(f"latent_prepare.x: shape {tuple(x.shape)} does not hold the queries and the low-rank part")
+    _chk(positions, "latent_prepare.positions", torch.int32, (n,))
+    _chk(tok_entry, "latent_prepare.tok_entry", torch.int32, (n,))
+    _chk(block_table, "latent_prepare.block_table", torch.int32)
+    _chk(norm_w, "latent_prepare.norm_w", torch.float32, (rank,))
+    _chk(q_out, "latent_prepare.q_out", None, (n, n_heads * dk))
+    if q_out.dtype != torch.float32 and x.dtype not in (torch.float32, q_out.dtype):
+        raise KernelError(f"latent_prepare: {x.dtype} inputs and {q_out.dtype} queries")
+    if q_out.dtype == torch.float32 and x.dtype != torch.float32:
+        raise KernelError("latent_prepare: float32 queries need float32 inputs")
+    rot = max_pos = 0
+    if cos is not None:
+        _chk(cos, "latent_prepare.cos", torch.float32)
+        _chk(sin, "latent_prepare.sin", torch.float32, cos.shape)
+        max_pos, half = cos.shape
+        rot = 2 * half
+        if rot > rot_dim:
+            raise KernelError(f"latent_prepare: {rot} rotated elements in a part of {rot_dim}")
+    _chk(k_pages, "latent_prepare.k_pages", q_out.dtype)
+    if k_pages.dim() != 4 or k_pages.shape[1] != 1 or k_pages.shape[3] != dk:
+        raise KernelError(f"latent_prepare.k_pages: shape {tuple(k_pages.shape)}, expected [pages, 1, page_size, {dk}]")
+    num_pages, _, page_size, _ = k_pages.shape
+    _chk(v_pages, "latent_prepare.v_pages", q_out.dtype, (num_pages, 1, rank, page_size))
+    _run(load_lib("vt_latent", half=_half(x, q_out)), "vt_latent_prepare", _ptr(x), _i(_code(x)),
+         ctypes.c_longlong(x.stride(0)), _i(q_column), _i(c_column), _ptr(norm_w), _f(eps), _ptr(cos), _ptr(sin), _i(rot),
+         _i(max_pos), _ptr(positions), _ptr(tok_entry), _ptr(block_table), _i(block_table.shape[1]), _ptr(q_out),
+         _ptr(k_pages), _ptr(v_pages), _i(_code(q_out)), _i(page_size), _i(num_pages), _i(n), _i(n_heads), _i(plain_dim),
+         _i(rot_dim), _i(rank), _stream())
+
+
+def head_linear(x: torch.Tensor, x_column: int, x_head: int, w: torch.Tensor, transposed: bool, y: torch.Tensor,
+                y_column: int, y_head: int, n_heads: int, n_in: int, n_out: int, gate: Optional[torch.Tensor] = None,
+                gate_column: int = 0) -> torch.Tensor:
+    """One small matrix per head: y[t, y_column + h * y_head + o] = sum_i W_h[o, i] x[t, x_column + h * x_head + i]
+    (w [H * n_out, n_in]), or with `transposed` sum_i W_h[i, o] x[...] (w [H * n_in, n_out]); times
+    sigmoid(gate[t, gate_column + h * n_out + o]) if `gate` is given.  x and y are 2-d tensors whose rows are the
+    tokens'; float32 sums.  16-bit inputs go to the matrix cores."""
+    n = x.shape[0]
+    _chk(x, "head_linear.x")
+    _chk(y, "head_linear.y")
+    _chk(w, "head_linear.w", y.dtype, (n_heads * (n_in if transposed else n_out), n_out if transposed else n_in))
+    if x.dim() != 2 or y.dim() != 2 or y.shape[0] != n:
+        raise KernelError("head_linear: x and y are [tokens, columns]")
+    if x_column < 0 or x.shape[1] < x_column + (n_heads - 1) * x_head + n_in or x_head < 0:
+        raise KernelError(f"head_linear.x: shape {tuple(x.shape)} has no {n_heads} heads of {n_in} from column {x_column}")
+    if y_column < 0 or y.shape[1] < y_column + (n_heads - 1) * y_head + n_out or y_head < n_out:
+        raise KernelError(f"head_linear.y: shape {tuple(y.shape)} has no {n_heads} heads of {n_out} from column {y_column}")
+    if n_in > HEAD_LINEAR_MAX_IN:
+        raise KernelError(f"head_linear: {n_in} inputs per head (up to {HEAD_LINEAR_MAX_IN})")
+    if y.dtype == torch.float32 and x.dtype != torch.float32:
+        raise KernelError("head_linear: float32 results need float32 inputs")
+    gptr, gcode, ldg = ctypes.c_void_p(0), F32, 0
+    if gate is not None:
+        _chk(gate, "head_linear.gate")
+        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads * n_out:
+            raise KernelError(f"head_linear.gate: shape {tuple(gate.shape)} has no {n_heads * n_out} columns from {gate_column}")
+        if y.dtype == torch.float32 and gate.dtype != torch.float32:
+            raise KernelError("head_linear: float32 results take float32 gates")
+        gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
+        gcode, ldg = _code(gate), gate.stride(0)
+    xptr = ctypes.c_void_p(x.data_ptr() + x_column * x.element_size())
+    yptr = ctypes.c_void_p(y.data_ptr() + y_column * y.element_size())
+    cores = (x.dtype in LOWP and n_in % 4 == 0 and x_head % 4 == 0 and x.stride(0) % 4 == 0 and x_column % 4 == 0)
+    _run(load_lib("vt_latent", half=_half(x, y, gate)), "vt_head_linear", xptr, _i(_code(x)), ctypes.c_longlong(x.stride(0)),
+         _i(x_head), _ptr(w), gptr, _i(gcode), ctypes.c_longlong(ldg), yptr, _i(_code(y)), ctypes.c_longlong(y.stride(0)),
+         _i(y_head), _i(n), _i(n_heads), _i(n_in), _i(n_out), _i(1 if transposed else 0), _i(1 if cores else 0), _stream())
+    return y
 
 
 # ---------------------------------------------------------------------------

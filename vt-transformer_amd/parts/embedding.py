@@ -42,8 +42,13 @@ class TokenEmbedding(Part):
 class LinearHead(Part):
     replayable = True
 
-    def __init__(self, *, rt: Runtime, width: int, vocab_size: int, name: str, tied_to: Optional[str] = None):
+    def __init__(self, *, rt: Runtime, width: int, vocab_size: int, name: str, tied_to: Optional[str] = None,
+                 softcap: float = 0.0):
+        """softcap: c > 0 bounds the logits to (-c, c): logits <- c tanh(logits / c)."""
         self.rt, self.width, self.vocab, self.name, self.tied_to = rt, int(width), int(vocab_size), name, tied_to
+        self.softcap = float(softcap or 0.0)
+        if self.softcap < 0:
+            raise ValueError("softcap must not be negative (0: the logits are not bounded)")
         self.weight: Optional[torch.Tensor] = None
         self.packed = None
 
@@ -69,10 +74,11 @@ class LinearHead(Part):
         r = x.shape[0]
         out = self.rt.buffer("logits", (r, self.vocab), torch.float32)
         if self.rt.dtype == torch.float32:
-            return ops.linear_f32(x, self.weight, None, out)
+            ops.linear_f32(x, self.weight, None, out)
+            return ops.tanh_cap(out, self.softcap) if self.softcap > 0 else out
         for r0 in range(0, r, SKINNY_MAX_ROWS):
             r1 = min(r, r0 + SKINNY_MAX_ROWS)
             need = ops.linear_bf16_workspace(r1 - r0, self.vocab, self.width) if r1 - r0 > 16 else 0
             work = self.rt.buffer("linear.partials", (need,), torch.float32) if need else None
             ops.linear_bf16(x[r0:r1], self.packed, None, out[r0:r1], work)
-        return out
+        return ops.tanh_cap(out, self.softcap) if self.softcap > 0 else out

@@ -1,4 +1,4 @@
-"""Gated feed-forward: down( act(gate(x)) * up(x) ), no biases.
+"""Gated feed-forward: down( act(gate(x)) * up(x) ).
 
 The reference's order (v1/models/qwen2-7b/inference_fp16.dag:333-337): up
 projection (mlp.w2), gate projection (mlp.w1), silu(gate) * up
@@ -7,6 +7,14 @@ projection (mlp.w2), gate projection (mlp.w1), silu(gate) * up
 (v1/models/qwen2-7b/dump_from_huggingface.py:89-99).  Gate and up are one
 matrix here (gate rows, then up rows); with few tokens the gating is applied
 to the fp32 accumulators inside the product's kernel.
+
+The gate's form has parameters: with g = gate(x) and u = up(x), both with their
+biases if the model has them,
+
+    g <- min(g, limit),  u <- clamp(u, -limit, limit)        (limit 0: no bounds)
+    act = g * sigmoid(alpha * g) * (u + up_shift)
+
+alpha 1, no bounds and no shift is SiLU gating, the reference's.
 """
 from __future__ import annotations
 
@@ -25,11 +33,20 @@ class GatedMLP(Part):
     replayable = True
 
     def __init__(self, *, rt: Runtime, width: int, prefix: str, intermediate_size: int, activation: str = "silu",
-                 names: Optional[Dict[str, str]] = None, weight_suffix: str = ".weight"):
+                 names: Optional[Dict[str, str]] = None, weight_suffix: str = ".weight",
+                 bias_suffix: Optional[str] = None, act_alpha: float = 1.0, act_limit: float = 0.0, up_shift: float = 0.0):
         """names: the three matrices' names behind the prefix; weight_suffix: what follows a matrix's name in its
-        tensor's name ("" where the tensor is called as the matrix)."""
+        tensor's name ("" where the tensor is called as the matrix); bias_suffix: likewise for the three biases
+        (None: the projections have none); act_alpha, act_limit, up_shift: the gate's form (module docstring)."""
         if activation != "silu":
-            raise ValueError(f"activation '{activation}' is not supported (only 'silu')")
+            raise ValueError(f"activation '{activation}' is not supported (only 'silu', whose form act_alpha, act_limit "
+                             f"and up_shift change)")
+        if not act_alpha > 0 or act_limit < 0:
+            raise ValueError("act_alpha must be positive and act_limit not negative (0: no bounds)")
+        self.alpha, self.limit, self.shift = float(act_alpha), float(act_limit), float(up_shift)
+        self.plain_silu = self.alpha == 1.0 and self.limit == 0.0 and self.shift == 0.0
+        self.bias_suffix = bias_suffix
+        self.b_gu = self.b_gu_lowp = self.b_down = self.b_down_lowp = None
         self.rt = rt
         self.width = int(width)
         self.inter = int(intermediate_size)
@@ -37,23 +54,39 @@ class GatedMLP(Part):
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
         self.suffix = weight_suffix
-        self.w_gu = self.w_down = self.p_gu = self.p_down = None
+        self.w_gu = self.w_down = self.p_gu = self.p_gu_plain = self.p_down = None
 
     def tensors(self) -> Dict[str, TensorDecl]:
         nm = self.names
-        return {
+        t = {
             nm["gate"] + self.suffix: TensorDecl((self.inter, self.width), "matrix"),
             nm["up"] + self.suffix: TensorDecl((self.inter, self.width), "matrix"),
             nm["down"] + self.suffix: TensorDecl((self.width, self.inter), "matrix"),
         }
+        if self.bias_suffix is not None:
+            t[nm["gate"] + self.bias_suffix] = TensorDecl((self.inter,), "bias")
+            t[nm["up"] + self.bias_suffix] = TensorDecl((self.inter,), "bias")
+            t[nm["down"] + self.bias_suffix] = TensorDecl((self.width,), "bias")
+        return t
 
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
         nm = self.names
         self.w_gu = torch.cat([rt.place(get(nm["gate"] + self.suffix), "matrix"),
                                rt.place(get(nm["up"] + self.suffix), "matrix")], dim=0).contiguous()
         self.w_down = rt.place(get(nm["down"] + self.suffix), "matrix")
-        self.p_gu, self.p_down = rt.pack(self.w_gu, halves=2), rt.pack(self.w_down)
-        self.w_gu, self.w_down = rt.row_major(self.w_gu, self.p_gu), rt.row_major(self.w_down, self.p_down)
+        if self.bias_suffix is not None:
+            self.b_gu = torch.cat([rt.place(get(nm["gate"] + self.bias_suffix), "bias"),
+                                   rt.place(get(nm["up"] + self.bias_suffix), "bias")], dim=0).contiguous()
+            self.b_down = rt.place(get(nm["down"] + self.bias_suffix), "bias")
+            self.b_gu_lowp, self.b_down_lowp = self.b_gu.to(rt.dtype), self.b_down.to(rt.dtype)
+        self.p_down = rt.pack(self.w_down)
+        if self.plain_silu and self.b_gu is None:
+            self.p_gu = rt.pack(self.w_gu, halves=2)       # gate and up side by side for the kernel that gates on its way
+            self.w_gu = rt.row_major(self.w_gu, self.p_gu)
+        else:
+            self.p_gu_plain = rt.pack(self.w_gu)           # one matrix of 2 I rows for the plain product
+            self.w_gu = rt.row_major(self.w_gu, self.p_gu_plain)
+        self.w_down = rt.row_major(self.w_down, self.p_down)
 
     takes_normed_input = True     # the gate/up product applies the norm in front of it when the rows are few
     hands_norm_on = True          # ... and the down product prepares the norm behind it
@@ -66,6 +99,13 @@ class GatedMLP(Part):
         rt = self.rt
         n = x.shape[0]
         act = rt.buffer("mlp.act", (n, self.inter), rt.dtype)
+        if not self.plain_silu or self.b_gu is not None:
+            # another form of the gate, or biases: the product (which takes the norm in front of it where it can), the
+            # gate as a kernel of its own, the down product
+            gu = linear(rt, x, self.w_gu, self.b_gu, "mlp.gu", bias_lowp=self.b_gu_lowp, packed=self.p_gu_plain)
+            ops.gated_act(gu, act, self.alpha, self.limit, self.shift)
+            return linear(rt, act, self.w_down, self.b_down, "mlp.down", bias_lowp=self.b_down_lowp, packed=self.p_down,
+                          residual=residual, hand_on=hand_on)
         normed = isinstance(x, NormedInput)
         if normed:
             ok = (takes_prepared_norm(rt, n, self.width) and self.p_gu is not None) if x.prepared else \

@@ -1,17 +1,27 @@
 """Attention mixer for heads that `PagedAttention`'s kernels do not take: keys
 and values of different sizes, rotation of part of the head, queries and
-keys scaled to unit root mean square, scores capped by a tanh, keys masked by
-a window or by chunks of positions, and one sigmoid gate per head on the
-output.  Every one of these is a constructor parameter that can be left out.
+keys scaled to unit root mean square, queries that grow with the logarithm of
+the position, scores capped by a tanh or lowered by a slope times the
+distance, keys masked by a window or by chunks of positions, a learned sink in
+the softmax's denominator, values mixed with those of an earlier layer, and
+one sigmoid gate per head on the output.  Every one of these is a constructor
+parameter that can be left out.
 
 Per token: q, k, v (and the gates' logits) in one matrix product with the
 biases; rotation, unit scaling and the write into the pages in one kernel;
 scores, cap, mask, float32 softmax, weighted sum and gate in one kernel that
 reads the pages; output projection.
 
-    score(i, j) = cap * tanh(scale * q_i . k_j / cap)                 (cap 0: scale * q_i . k_j)
+    q_i = temp(i) * (W_q x_i),  temp(i) = 1 + coef * ln(floor((i + 1) / every) + 1)           (no q_temp: 1)
+    score(i, j) = cap * tanh(scale * q_i . k_j / cap) - slope_h * (i - j)                     (cap 0: scale * q_i . k_j)
+    slope_h = 2^(-distance_slopes * (h + 1) / H)                                              (no distance_slopes: 0)
     j is seen from i  <=>  j <= i,  i - j < window (if window > 0),  floor(j / chunk) = floor(i / chunk) (if chunk > 0)
-    out_i[h] = sigmoid(gate_i[h]) * sum_j softmax_j(score(i, j)) v_j
+    p_ij = exp(score(i, j)) / (sum_j' exp(score(i, j')) + exp(sink_h))                        (no sink: the plain softmax)
+    out_i[h] = sigmoid(gate_i[h]) * sum_j p_ij v_j
+
+Value mixing ties layers together: the first layer of a model that says value_mix="source" leaves the step's values
+in a buffer, and every layer that says value_mix="mix" keeps (1 - lambda) v + lambda v_source in its pages instead
+of its own v, with lambda a learned number of its own.
 
 Chunks are counted from position 0 of the sequence.  A key that no later
 position can see is dead for the cache manager: the pages' window is the
@@ -31,6 +41,29 @@ from .base import MIXERS, POSITIONS, CacheNeed, PageTensor, Part, Runtime, State
 from .linear import linear
 
 
+TILE_ROWS = 16
+TILES_KEY = ("masked_attention.tiles", TILE_ROWS)
+
+
+def plan_tiles(ctx) -> Optional[Dict[tuple, np.ndarray]]:
+    """The work of `ops.attention_masked_mfma` for a step that brings more than single tokens: runs of up to 16
+    consecutive tokens of one request, (first row, rows).  One list serves every layer whose mixer goes through that
+    kernel; it is found as ctx.extra[TILES_KEY]."""
+    if ctx.single_token or TILES_KEY in ctx.extra_host:
+        return None
+    start = np.asarray(ctx.h_entry_start, dtype=np.int64)
+    tiles = []
+    for e in range(len(start) - 1):
+        for first in range(int(start[e]), int(start[e + 1]), TILE_ROWS):
+            tiles.append((first, min(TILE_ROWS, int(start[e + 1]) - first)))
+    return {TILES_KEY: np.asarray(tiles, dtype=np.int32).reshape(-1)}
+
+
+def head_slopes(n_heads: int, steepness: float) -> np.ndarray:
+    """slope_h = 2^(-steepness (h + 1) / H), float32."""
+    return np.power(2.0, -float(steepness) * (np.arange(n_heads, dtype=np.float64) + 1.0) / n_heads).astype(np.float32)
+
+
 @MIXERS.register("masked_attention")
 class MaskedAttention(Part):
     replayable = True       # a decoding step's launches depend on the number of entries only
@@ -39,13 +72,17 @@ class MaskedAttention(Part):
                  value_dim: Optional[int] = None, qkv_bias: bool = False, position: Optional[PartSpec] = None,
                  scale: Optional[float] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0,
                  unit_rms_eps: Optional[float] = None, head_gate: bool = False, shared: Optional[dict] = None,
-                 names: Optional[Dict[str, str]] = None):
+                 names: Optional[Dict[str, str]] = None, sink: bool = False, distance_slopes: Optional[float] = None,
+                 q_temp: Optional[Dict[str, float]] = None, value_mix: Optional[str] = None):
         """key_dim / value_dim: sizes of a head's queries and keys / of its values (default: the same);
         position: a rotary encoding whose `dim` may be smaller than key_dim (the rest of a head passes unchanged);
         unit_rms_eps: queries and keys are divided by their root mean square per head after the rotation, with
         this eps inside the root (None: they are not); head_gate: one sigmoid gate per head from a projection of
-        the mixer's input; names: tensor names behind the prefix for q, k, v, o, g and the biases q_bias, k_bias,
-        v_bias."""
+        the mixer's input; names: tensor names behind the prefix for q, k, v, o, g, sink, vmix and the biases q_bias,
+        k_bias, v_bias; sink: one learned number per head whose exponential joins the softmax's denominator;
+        distance_slopes: s > 0 takes 2^(-s (h + 1) / H) times the distance off head h's scores; q_temp {coef, every}:
+        the queries' factor by position; value_mix: "source" (this layer's values are what later layers mix in),
+        "mix" (this layer keeps (1 - lambda) v + lambda v_source, lambda its tensor `vmix`) or None."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
         self.rt, self.width = rt, int(width)
@@ -60,8 +97,20 @@ class MaskedAttention(Part):
         if self.softcap < 0 or self.window < 0 or self.chunk < 0:
             raise ValueError("softcap, window and chunk must not be negative (0 switches each off)")
         self.unit_rms_eps = None if unit_rms_eps is None else float(unit_rms_eps)
+        self.has_sink = bool(sink)
+        self.distance_slopes = None if not distance_slopes else float(distance_slopes)
+        if self.distance_slopes is not None and self.distance_slopes < 0:
+            raise ValueError("distance_slopes must be positive (None switches the slopes off)")
+        self.q_temp = None
+        if q_temp:
+            self.q_temp = (float(q_temp["coef"]), int(q_temp["every"]))
+            if self.q_temp[1] <= 0:
+                raise ValueError(f"q_temp.every {self.q_temp[1]} must be positive")
+        if value_mix not in (None, "source", "mix"):
+            raise ValueError(f"value_mix {value_mix!r} ('source', 'mix' or None)")
+        self.value_mix = value_mix
         n = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "g": "g_proj.weight",
-             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias"}
+             "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "sink": "sink", "vmix": "vmix"}
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
         pos_spec = position or PartSpec("none", {})
@@ -75,6 +124,7 @@ class MaskedAttention(Part):
         if getattr(self.position, "dim", 0) and not hasattr(self.position, "rotary_tables"):
             raise ValueError("this mixer takes rotary position encodings (or none)")
         self.w_in = self.b_in = self.b_in_lowp = self.p_in = self.w_o = self.p_o = None
+        self.sink = self.slopes = self.v_lambda = None
 
     # columns of the input projection: queries, keys, values, gates
     @property
@@ -93,22 +143,13 @@ class MaskedAttention(Part):
         """Whether portions of prompts go to the matrix-core kernel: a 16-bit runtime and heads in multiples of 16."""
         return self.rt.lowp and ops.attention_masked_mfma_takes(self.d, self.dv, 16)
 
-    TILE_ROWS = 16
+    TILE_ROWS = TILE_ROWS
 
     def prepare_step(self, ctx) -> Optional[Dict[tuple, np.ndarray]]:
-        """The matrix-core kernel's work for a step that brings more than single tokens: runs of up to 16 consecutive
-        tokens of one request, (first row, rows).  One list serves every layer of this kind."""
-        if not self._matrix_cores() or ctx.single_token:
+        """The matrix-core kernel's work for a step that brings more than single tokens (`plan_tiles`)."""
+        if not self._matrix_cores():
             return None
-        key = ("masked_attention.tiles", self.TILE_ROWS)
-        if key in ctx.extra_host:
-            return None
-        start = np.asarray(ctx.h_entry_start, dtype=np.int64)
-        tiles = []
-        for e in range(len(start) - 1):
-            for first in range(int(start[e]), int(start[e + 1]), self.TILE_ROWS):
-                tiles.append((first, min(self.TILE_ROWS, int(start[e + 1]) - first)))
-        return {key: np.asarray(tiles, dtype=np.int32).reshape(-1)}
+        return plan_tiles(ctx)
 
     def state_need(self) -> Optional[StateNeed]:
         return None
@@ -127,6 +168,11 @@ class MaskedAttention(Part):
             t[nm["v_bias"]] = TensorDecl((self.nkv * self.dv,), "bias")
         if self.head_gate:
             t[nm["g"]] = TensorDecl((self.nh, self.width), "matrix")
+        if self.has_sink:
+            t[nm["sink"]] = TensorDecl((self.nh,), "bias")
+        if self.value_mix is not None:
+            # (the source layer's number is part of the checkpoint and is not used)
+            t[nm["vmix"]] = TensorDecl((), "bias", optional=self.value_mix == "source")
         return t
 
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
@@ -140,6 +186,12 @@ class MaskedAttention(Part):
             self.b_in = torch.cat(b, dim=0).contiguous()
             self.b_in_lowp = self.b_in.to(rt.dtype)
         self.w_o = rt.place(get(nm["o"]), "matrix")
+        if self.has_sink:
+            self.sink = rt.place(get(nm["sink"]), "bias")
+        if self.distance_slopes is not None:
+            self.slopes = torch.from_numpy(head_slopes(self.nh, self.distance_slopes)).to(rt.device)
+        if self.value_mix == "mix":
+            self.v_lambda = rt.place(get(nm["vmix"]), "bias").reshape(1)
         self.p_in, self.p_o = rt.pack(self.w_in), rt.pack(self.w_o)
         self.w_in, self.w_o = rt.row_major(self.w_in, self.p_in), rt.row_major(self.w_o, self.p_o)
 
@@ -152,16 +204,20 @@ class MaskedAttention(Part):
         tables = self.position.rotary_tables(ctx.n_positions) if getattr(self.position, "dim", 0) else None
         cos, sin = tables if tables is not None else (None, None)
         q = rt.buffer("mattn.q", (n, nh * d), rt.dtype)
+        # the values that layers mix: one buffer per model and step, written by the source layer, read by the others
+        v_first = rt.buffer("mattn.v_first", (n, nkv * dv), torch.float32) if self.value_mix is not None else None
         ops.qk_prepare(y, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, nkv,
-                       d, dv, self.unit_rms_eps)
+                       d, dv, self.unit_rms_eps, q_temp=self.q_temp, v_first=v_first, v_lambda=self.v_lambda)
         out = rt.buffer("mattn.out", (n, nh * dv), rt.dtype)
-        tiles = ctx.extra.get(("masked_attention.tiles", self.TILE_ROWS)) if self._matrix_cores() and not ctx.single_token else None
+        tiles = ctx.extra.get(TILES_KEY) if self._matrix_cores() and not ctx.single_token else None
         if tiles is not None and cache["k"].shape[2] % 16 == 0:
             ops.attention_masked_mfma(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, tiles, out,
                                       nh, nkv, d, dv, self.scale, self.softcap, self.window, self.chunk,
-                                      gate=y if self.head_gate else None, gate_column=self._gate_column)
+                                      gate=y if self.head_gate else None, gate_column=self._gate_column,
+                                      sink=self.sink, slopes=self.slopes)
             return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o)
         ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
                              dv, self.scale, self.softcap, self.window, self.chunk,
-                             gate=y if self.head_gate else None, gate_column=self._gate_column)
+                             gate=y if self.head_gate else None, gate_column=self._gate_column,
+                             sink=self.sink, slopes=self.slopes)
         return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o)
