@@ -192,6 +192,25 @@ def pair_configs(key: str, chunk: int):
     return lis, qwen
 
 
+def gabelorn_pair_configs(key: str, window: int):
+    """(Gabelorn config.json, Qwen2 config.json) of equal sizes: latent-attention and slope-attention layers in turn,
+    a feed-forward behind each.  The latent layers keep 192 + 64 numbers per token (the attention kernels' largest
+    key) and see `window` positions; the attention layers have Qwen2's heads and see every key."""
+    width, layers, heads, kv, d, ff, vocab = PAIR_SIZES[key]
+    mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+    latent = {"type": "latent_attention", "mlp": mlp,
+              "mixer": {"heads": heads, "dim": d, "rot_dim": 64, "vdim": d, "kv_rank": 192, "scale": (d + 64) ** -0.5,
+                        "mask": {"size": window}, "rot": {"dims": 64, "base": 1e6}}}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": heads, "kv_heads": kv, "dim": d, "vdim": d, "scale": d ** -0.5,
+                     "q_temp": {"coef": 0.1, "every": 1024}, "v_mix": True}}
+    gab = {"architecture": "Gabelorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_softcap": 30.0,
+           "layers": [latent if i % 2 == 0 else att for i in range(layers)], "max_positions": 32768}
+    qwen = dict(QWEN2_7B, vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
+                num_attention_heads=heads, num_key_value_heads=kv, head_dim=d, max_position_embeddings=32768)
+    return gab, qwen
+
+
 class PairBench(Bench):
     """Bench's measurements on an engine built from any config.json."""
 
@@ -213,42 +232,44 @@ class PairBench(Bench):
         print(f"[bench] {name}: model ready in {time.time() - t0:.1f} s", file=sys.stderr, flush=True)
 
 
-def lisunex_pairs(args) -> int:
-    """Prefill and decode of Lisunex beside Qwen2 at equal sizes; one JSON line."""
-    keys = [k.strip() for k in args.lisunex.split(",") if k.strip()]
+def design_pairs(args, design: str) -> int:
+    """Prefill and decode of a second design (lisunex or gabelorn) beside Qwen2 at equal sizes; one JSON line."""
+    title = design.capitalize()
+    keys = [k.strip() for k in getattr(args, design).split(",") if k.strip()]
     for k in keys:
         if k not in PAIR_SIZES:
-            print(f"bench.py: --lisunex takes {', '.join(PAIR_SIZES)}; got '{k}'")
+            print(f"bench.py: --{design} takes {', '.join(PAIR_SIZES)}; got '{k}'")
             return 2
     T, batch, prompt_len = args.prefill_tokens, args.batch, args.prompt_len or 1024
     per_req = -(-(prompt_len + args.steps + args.warmup + 32) // 16) * 16
     pool = max(batch * per_req, T + 64)
+    span = args.lisunex_chunk if design == "lisunex" else args.gabelorn_window
     out = {}
     for k in keys:
-        lis, qwen = pair_configs(k, args.lisunex_chunk)
+        other, qwen = pair_configs(k, span) if design == "lisunex" else gabelorn_pair_configs(k, span)
         row = {}
-        for name, cfg_d in (("lisunex", lis), ("qwen2", qwen)):
+        for name, cfg_d in ((design, other), ("qwen2", qwen)):
             b = PairBench(f"{name} {k}", cfg_d, args.dtype, batch, pool, max(pool // batch, T + 64) + 64, graphs=not args.no_graphs)
             p_dt = b.prefill_run(T)
             tps, ms, _ = b.decode_run(batch, args.steps, args.warmup, prompt_len)
             row[name] = {"prefill_tok_s": round(T / p_dt, 1), "prefill_ms": round(p_dt * 1e3, 3),
                          "decode_tok_s": round(tps, 1), "decode_ms_per_step": round(ms, 4)}
             b.close()
-        row["lisunex_over_qwen2"] = {"prefill": round(row["lisunex"]["prefill_tok_s"] / row["qwen2"]["prefill_tok_s"], 3),
-                                     "decode": round(row["lisunex"]["decode_tok_s"] / row["qwen2"]["decode_tok_s"], 3)}
+        row[f"{design}_over_qwen2"] = {"prefill": round(row[design]["prefill_tok_s"] / row["qwen2"]["prefill_tok_s"], 3),
+                                       "decode": round(row[design]["decode_tok_s"] / row["qwen2"]["decode_tok_s"], 3)}
         width, layers, heads, kv, d, ff, vocab = PAIR_SIZES[k]
         row["sizes"] = f"L{layers} H{width} NH{heads} KVH{kv} D{d} I{ff} V{vocab}"
         out[k] = row
     first = out[keys[0]]
     print(json.dumps({
-        "metric": f"Lisunex decode tok/s at batch {batch} after {prompt_len:,}-token prompts, sizes {keys[0]} "
+        "metric": f"{title} decode tok/s at batch {batch} after {prompt_len:,}-token prompts, sizes {keys[0]} "
                   f"(beside Qwen2 at equal sizes; prefill of {T:,} tokens under `pairs`)",
-        "value": first["lisunex"]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": first["lisunex"]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "value": first[design]["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": first[design]["decode_ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": {"bfloat16": "bf16", "float16": "fp16"}[args.dtype],
         "data": "synthetic (random weights N(0,0.02), uniform random token ids)",
-        "config": {"model": "Lisunex and Qwen2 at equal sizes", "global_batch": batch, "seq_len": prompt_len,
-                   "prefill_tokens": T, "chunk": args.lisunex_chunk, "parallelism": "1 GPU"},
+        "config": {"model": f"{title} and Qwen2 at equal sizes", "global_batch": batch, "seq_len": prompt_len,
+                   "prefill_tokens": T, "chunk" if design == "lisunex" else "window": span, "parallelism": "1 GPU"},
         "pairs": out}), flush=True)
     return 0
 
@@ -296,15 +317,20 @@ def main() -> int:
                          "Qwen2 at equal sizes, prefill of --prefill-tokens and decode at --batch; sizes by name, "
                          "with commas: " + ", ".join(PAIR_SIZES))
     ap.add_argument("--lisunex-chunk", type=int, default=1024, help="positions per chunk of Lisunex's attention mask")
+    ap.add_argument("--gabelorn", default="", metavar="SIZES",
+                    help="another workload instead: the Gabelorn design (latent-attention and slope-attention layers in "
+                         "turn) beside Qwen2 at equal sizes, prefill of --prefill-tokens and decode at --batch; sizes by "
+                         "name, with commas: " + ", ".join(PAIR_SIZES))
+    ap.add_argument("--gabelorn-window", type=int, default=1024, help="positions that a latent-attention layer sees")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; N > 1 is not measured")
         return 2
 
-    if args.lisunex:
+    if args.lisunex or args.gabelorn:
         if args.dtype == "float16":
-            args.dtype = "bfloat16"         # the serving dtype of this design
-        return lisunex_pairs(args)
+            args.dtype = "bfloat16"         # the serving dtype of these designs
+        return design_pairs(args, "lisunex" if args.lisunex else "gabelorn")
 
     import torch
 

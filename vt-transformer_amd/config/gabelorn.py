@@ -180,7 +180,7 @@ class GabelornConfig(ModelConfig):
             "num_heads": int(m["heads"]), "num_kv_heads": int(m["kv_heads"]), "key_dim": int(m["dim"]),
             "value_dim": int(m["vdim"]), "scale": float(m["scale"]), "sink": True, "distance_slopes": SLOPE_STEEPNESS,
             "q_temp": {"coef": float(qt["coef"]), "every": int(qt["every"])} if qt else None, "value_mix": value_mix,
-            "names": dict(_ATTENTION_NAMES), "prefix": "mix.",
+            "fuse_norms": True, "names": dict(_ATTENTION_NAMES), "prefix": "mix.",
         })
 
     def to_spec(self) -> ModelSpec:

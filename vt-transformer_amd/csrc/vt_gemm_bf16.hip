@@ -137,6 +137,19 @@ __device__ __forceinline__ bf16x8_t load_x(const bf16_t* row, int k, int K) {
 // block order and multiplies its sums by 1/sqrt(sum / width + eps), which is where the norm's division belongs
 // since it is the same for a whole row.  The shares are added in a fixed order: the result does not depend on
 // which block finished first.  Rows of ssq are SSQ_STRIDE(N) floats apart.
+// The form of the gated product's gate, with g and u the two matrices' sums (and their biases, if any):
+//     g <- min(g, limit), u <- clamp(u, -limit, limit)   (limit 0: no bounds);   g * sigmoid(alpha * g) * (u + shift).
+// alpha 1, limit 0, shift 0 is SiLU gating, to the bit what it was before the form had parameters.
+struct GateForm {
+    float alpha, limit, shift;
+};
+__device__ __forceinline__ float gate_form(float g, float u, const GateForm& f) {
+    if (f.limit > 0.f) {
+        g = fminf(g, f.limit);
+        u = fminf(fmaxf(u, -f.limit), f.limit);
+    }
+    return g / (1.f + expf(-f.alpha * g)) * (u + f.shift);
+}
 struct NormLink {
     bf16_t* xn_out;            // producer: [N][Mout], or null
     const float* gain_next;    //           [Mout]
@@ -144,6 +157,7 @@ struct NormLink {
     const float* ssq_in;       // consumer: [n_ssq][stride], or null
     int n_ssq;
     float eps;
+    GateForm gate;             // (rides along: the gate's form of a gated product)
 };
 #define SSQ_STRIDE(N) ((N) <= 16 ? 16 : 64)
 
@@ -444,8 +458,13 @@ __global__ __launch_bounds__(WPB * 64) void gemm_skinny_kernel(const void* __res
                 v *= rinv;
                 u *= rinv;
             }
-            if (SWIGLU) v = v / (1.f + expf(-v)) * u;
-            else if (bias) v += bias[m];
+            if (SWIGLU) {
+                if (bias) {
+                    v += bias[m];
+                    u += bias[Mout + m];
+                }
+                v = gate_form(v, u, link.gate);
+            } else if (bias) v += bias[m];
             if (resid) v += resid[(size_t)n * Mout + m];
             store_f32<TO>(y, (size_t)n * Mout + m, v);
             if (link.xn_out) {
@@ -640,7 +659,11 @@ __global__ __launch_bounds__((WM + 1) * 64) void gemm_mid_kernel(const bf16_t* _
                 if (SWIGLU) {
                     float u = acc[R + j][i][e];
                     if (consumes) u *= link_rinv[(i * 16 + r) & 63];
-                    v = v / (1.f + expf(-v)) * u;
+                    if (bias) {
+                        v += bias[m];
+                        u += bias[Mout + m];
+                    }
+                    v = gate_form(v, u, link.gate);
                 } else if (bias && blockIdx.z == 0) {
                     v += bias[m];
                 }
@@ -867,7 +890,7 @@ __device__ __forceinline__ float packed_at(const bf16_t* wp, int KT, int m, int 
 template <bool SWIGLU, typename TO>
 __global__ void gemm_plain_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
                                   const float* __restrict__ bias, TO* __restrict__ y, int N, int Mout, int K, int KT,
-                                  int up_tiles) {
+                                  int up_tiles, GateForm gate) {
     int m = blockIdx.x * blockDim.x + threadIdx.x, n = blockIdx.y;
     if (m >= Mout) return;
     const bf16_t* xr = x + (size_t)n * K;
@@ -875,7 +898,11 @@ __global__ void gemm_plain_kernel(const bf16_t* __restrict__ x, const bf16_t* __
     for (int k = 0; k < K; ++k) v = fmaf(bf16_to_f32(xr[k]), packed_at(wp, KT, m, k), v);
     if (SWIGLU) {
         for (int k = 0; k < K; ++k) u = fmaf(bf16_to_f32(xr[k]), packed_at(wp, KT, up_tiles * 16 + m, k), u);
-        v = v / (1.f + expf(-v)) * u;
+        if (bias) {
+            v += bias[m];
+            u += bias[Mout + m];
+        }
+        v = gate_form(v, u, gate);
     } else if (bias) {
         v += bias[m];
     }
@@ -967,7 +994,7 @@ extern "C" long long vt_linear_bf16_workspace(int N, int M, int K, int gated) {
 
 // gain != null: x is the fp32 residual stream and the RMSNorm (gain, eps) is part of the product (up to 16 tokens);
 // resid != null: the result is added to it (up to 64 tokens).
-static const NormLink NO_LINK = {nullptr, nullptr, nullptr, nullptr, 0, 0.f};
+static const NormLink NO_LINK = {nullptr, nullptr, nullptr, nullptr, 0, 0.f, {1.f, 0.f, 0.f}};
 
 // shares of the rows' sums of squares that a producing product of this shape writes (0: it cannot produce)
 extern "C" int vt_linear_bf16_link_shares(int N, int M, int K) {
@@ -1001,7 +1028,7 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
     VT_REQUIRE((((uintptr_t)wp) & 15) == 0, "vt_linear_bf16: the packed matrix is not 16-byte aligned");
     if (K % 8 != 0 || ((uintptr_t)x & 15)) {
         VT_REQUIRE(N <= 65535, "vt_linear_bf16: too many rows (%d) for the any-shape kernel", N);
-        gemm_plain_kernel<SWIGLU, TO><<<dim3((Mout + 255) / 256, N), 256, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles);
+        gemm_plain_kernel<SWIGLU, TO><<<dim3((Mout + 255) / 256, N), 256, 0, stream>>>(x, wp, bias, y, N, Mout, K, KT, up_tiles, link.gate);
         VT_CHECK_LAUNCH("vt_linear_bf16(plain)");
         return 0;
     }
@@ -1032,7 +1059,7 @@ static int linear_bf16(const void* xv, const bf16_t* wp, const float* bias, TO* 
         VT_REQUIRE(!link.ssq_in || grid.y == 1, "vt_linear_bf16: a prepared norm is taken with up to 64 rows (N=%d)", N);
         // the product takes the norm in front (link.ssq_in); the one behind is prepared where the sums are added up
         NormLink in = NO_LINK;
-        in.ssq_in = link.ssq_in; in.n_ssq = link.n_ssq; in.eps = link.eps;
+        in.ssq_in = link.ssq_in; in.n_ssq = link.n_ssq; in.eps = link.eps; in.gate = link.gate;
 #define VT_MID__(W, O, T) do { \
             static bool lds_set = false; \
             if (!lds_set) { \
@@ -1167,7 +1194,7 @@ extern "C" int vt_linear_bf16_link(const void* x, const void* wp, const float* b
                                    void* xn_out, const float* gain_next, float* ssq_out, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && M > 0 && K > 0, "vt_linear_bf16_link: bad sizes N=%d M=%d K=%d", N, M, K);
     VT_REQUIRE(ssq_in || xn_out, "vt_linear_bf16_link: neither end of a norm: use vt_linear_bf16");
-    const NormLink link = {(bf16_t*)xn_out, gain_next, ssq_out, ssq_in, n_ssq, eps_in};
+    const NormLink link = {(bf16_t*)xn_out, gain_next, ssq_out, ssq_in, n_ssq, eps_in, {1.f, 0.f, 0.f}};
     return linear_bf16<false, float>(x, (const bf16_t*)wp, bias, y, workspace, N, M, K, nullptr, 0.f, resid, stream, link);
 }
 
@@ -1176,10 +1203,27 @@ extern "C" int vt_gated_linear_bf16_link(const void* x, const void* wp, void* y,
                                          const float* ssq_in, int n_ssq, float eps_in, hipStream_t stream) {
     VT_REQUIRE(N >= 0 && I > 0 && K > 0, "vt_gated_linear_bf16_link: bad sizes N=%d I=%d K=%d", N, I, K);
     VT_REQUIRE(ssq_in, "vt_gated_linear_bf16_link: no sums of squares: use vt_gated_linear_bf16");
-    const NormLink link = {nullptr, nullptr, nullptr, ssq_in, n_ssq, eps_in};
+    const NormLink link = {nullptr, nullptr, nullptr, ssq_in, n_ssq, eps_in, {1.f, 0.f, 0.f}};
     if (out_dtype == VT_F32) return linear_bf16<true, float>(x, (const bf16_t*)wp, nullptr, (float*)y, nullptr, N, I, K, nullptr, 0.f, nullptr, stream, link);
     if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>(x, (const bf16_t*)wp, nullptr, (bf16_t*)y, nullptr, N, I, K, nullptr, 0.f, nullptr, stream, link);
     return vt_fail("vt_gated_linear_bf16_link: unknown out dtype %d", out_dtype);
+}
+
+// The gated product with biases and a gate of another form (GateForm): y[N, I] = gate(x . Wg^T + bias[0..I),
+// x . Wu^T + bias[I..2I)).  bias may be null.  One of: plain 16-bit tokens; gain != null: x is the fp32 residual
+// stream and rmsnorm(x; gain, eps) takes its place (up to 16 tokens); ssq_in != null: x is a norm that the product in
+// front has prepared (n_ssq, eps as above).
+extern "C" int vt_gated_linear_bf16_form(const void* x, const void* wp, const float* bias, void* y, int out_dtype, int N,
+                                         int I, int K, const float* gain, float eps, const float* ssq_in, int n_ssq,
+                                         float alpha, float limit, float shift, hipStream_t stream) {
+    VT_REQUIRE(N >= 0 && I > 0 && K > 0, "vt_gated_linear_bf16_form: bad sizes N=%d I=%d K=%d", N, I, K);
+    VT_REQUIRE(!(gain && ssq_in), "vt_gated_linear_bf16_form: a norm in front is applied here or was prepared, not both");
+    VT_REQUIRE(alpha > 0.f && limit >= 0.f, "vt_gated_linear_bf16_form: bad gate (alpha %g, limit %g)", alpha, limit);
+    const NormLink link = {nullptr, nullptr, nullptr, ssq_in, ssq_in ? n_ssq : 0, ssq_in ? eps : 0.f, {alpha, limit, shift}};
+    const float* g = ssq_in ? nullptr : gain;
+    if (out_dtype == VT_F32) return linear_bf16<true, float>(x, (const bf16_t*)wp, bias, (float*)y, nullptr, N, I, K, g, eps, nullptr, stream, link);
+    if (out_dtype == VT_BF16) return linear_bf16<true, bf16_t>(x, (const bf16_t*)wp, bias, (bf16_t*)y, nullptr, N, I, K, g, eps, nullptr, stream, link);
+    return vt_fail("vt_gated_linear_bf16_form: unknown out dtype %d", out_dtype);
 }
 
 // y[N, I] = silu(x . Wg^T) * (x . Wu^T); wp = Wg [I, K] packed, followed by Wu [I, K] packed.

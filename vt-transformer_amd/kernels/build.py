@@ -36,7 +36,7 @@ DEFAULT_HEAD_DIMS = list(range(16, 257, 16))
 # sources with the other conversion and the other matrix instruction); the float16 build's name ends in _f16.
 HALF_LIBS = ("vt_elementwise", "vt_gemm_bf16", "vt_attn_bf16", "vt_attn_masked", "vt_attn_masked_mfma", "vt_delta", "vt_latent")
 # the matrix-core kernel of the masked attention is built per (key size, value size) of a head
-DEFAULT_MASKED_DIMS = [(64, 64), (128, 128), (64, 96), (48, 80), (32, 48), (16, 16), (64, 32), (64, 16), (48, 32), (192, 128)]
+DEFAULT_MASKED_DIMS = [(64, 64), (128, 128), (64, 96), (48, 80), (32, 48), (16, 16), (64, 32), (64, 16), (48, 32), (256, 192)]
 
 
 class KernelBuildError(RuntimeError):

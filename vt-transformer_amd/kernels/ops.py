@@ -497,6 +497,43 @@ def gated_linear_bf16(x: torch.Tensor, w_gate_up, out: torch.Tensor, norm_gain: 
     return out
 
 
+def gated_linear_bf16_form(x: torch.Tensor, w: PackedMatrix, bias: Optional[torch.Tensor], out: torch.Tensor,
+                           alpha: float, limit: float, shift: float, norm_gain: Optional[torch.Tensor] = None,
+                           norm_eps: float = 0.0, ssq_in: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = gate(x Wg^T + bias[:I], x Wu^T + bias[I:]) with gate(g, u) = g' sigmoid(alpha g') (u' + shift),
+    g' = min(g, limit), u' = clamp(u, -limit, limit) (limit 0: no bounds); w: two packed halves.  x: 16-bit tokens;
+    or with norm_gain the float32 residual stream whose RMSNorm is what gets multiplied (up to 16 rows); or with
+    ssq_in a norm that the product in front has prepared (gated_linear_bf16_link's x and ssq_in, eps in norm_eps)."""
+    n, k = x.shape
+    lp = _lowp(w.data, "gated_linear_bf16_form.w")
+    if w.cols != k or w.halves != 2:
+        raise KernelError(f"gated_linear_bf16_form: x [{n}, {k}] does not fit a packed matrix [{w.rows}, {w.cols}] x {w.halves}")
+    if norm_gain is not None and ssq_in is not None:
+        raise KernelError("gated_linear_bf16_form: a norm in front is applied here or was prepared, not both")
+    _chk(x, "gated_linear_bf16_form.x", torch.float32 if norm_gain is not None else lp)
+    _chk(w.data, "gated_linear_bf16_form.w", lp)
+    _chk(out, "gated_linear_bf16_form.out", None, (n, w.rows))
+    if bias is not None:
+        _chk(bias, "gated_linear_bf16_form.bias", torch.float32, (2 * w.rows,))
+    if norm_gain is not None:
+        if n > 16 or k % 8:
+            raise KernelError(f"gated_linear_bf16_form: the fused norm takes at most 16 rows and k a multiple of 8 (n={n}, k={k})")
+        _chk(norm_gain, "gated_linear_bf16_form.norm_gain", torch.float32, (k,))
+    n_ssq = 0
+    if ssq_in is not None:
+        _chk(ssq_in, "gated_linear_bf16_form.ssq_in", torch.float32)
+        if n > 64 or ssq_in.dim() != 2 or ssq_in.shape[1] != link_stride(n):
+            raise KernelError(f"gated_linear_bf16_form: {n} rows, ssq_in of shape {tuple(ssq_in.shape)}: up to 64 rows and "
+                              f"[shares, {link_stride(n)}]")
+        n_ssq = ssq_in.shape[0]
+    if not alpha > 0 or limit < 0:
+        raise KernelError(f"gated_linear_bf16_form: gate with alpha {alpha} and limit {limit}")
+    _run(load_lib("vt_gemm_bf16", half=_half(w.data, x, out)), "vt_gated_linear_bf16_form", _ptr(x), _ptr(w.data), _ptr(bias),
+         _ptr(out), _i(_code(out)), _i(n), _i(w.rows), _i(k), _ptr(norm_gain), _f(norm_eps), _ptr(ssq_in), _i(n_ssq),
+         _f(alpha), _f(limit), _f(shift), _stream())
+    return out
+
+
 # ---------------------------------------------------------------------------
 def attention_f32(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, positions: torch.Tensor,
                   tok_entry: torch.Tensor, block_table: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int,

@@ -54,7 +54,7 @@ class GatedMLP(Part):
         n.update(names or {})
         self.names = {k: prefix + v for k, v in n.items()}
         self.suffix = weight_suffix
-        self.w_gu = self.w_down = self.p_gu = self.p_gu_plain = self.p_down = None
+        self.w_gu = self.w_down = self.p_gu = self.p_down = None
 
     def tensors(self) -> Dict[str, TensorDecl]:
         nm = self.names
@@ -80,12 +80,8 @@ class GatedMLP(Part):
             self.b_down = rt.place(get(nm["down"] + self.bias_suffix), "bias")
             self.b_gu_lowp, self.b_down_lowp = self.b_gu.to(rt.dtype), self.b_down.to(rt.dtype)
         self.p_down = rt.pack(self.w_down)
-        if self.plain_silu and self.b_gu is None:
-            self.p_gu = rt.pack(self.w_gu, halves=2)       # gate and up side by side for the kernel that gates on its way
-            self.w_gu = rt.row_major(self.w_gu, self.p_gu)
-        else:
-            self.p_gu_plain = rt.pack(self.w_gu)           # one matrix of 2 I rows for the plain product
-            self.w_gu = rt.row_major(self.w_gu, self.p_gu_plain)
+        self.p_gu = rt.pack(self.w_gu, halves=2)           # gate and up side by side for the kernel that gates on its way
+        self.w_gu = rt.row_major(self.w_gu, self.p_gu)
         self.w_down = rt.row_major(self.w_down, self.p_down)
 
     takes_normed_input = True     # the gate/up product applies the norm in front of it when the rows are few
@@ -95,17 +91,38 @@ class GatedMLP(Part):
         """Whether the down product adds to the residual stream itself at this many rows."""
         return can_add_residual(self.rt, rows, self.width, self.inter)
 
+    def _forward_formed(self, x, act, residual, hand_on):
+        """The gate in another form than SiLU's, or with biases.  Few rows in a 16-bit type: the gated product's kernel
+        takes biases and form (and the norm in front, as for SiLU).  Otherwise the plain product of both matrices
+        with the biases, the gate as a kernel of its own, and the down product."""
+        rt = self.rt
+        n = x.shape[0]
+        normed = isinstance(x, NormedInput)
+        if rt.lowp and self.p_gu is not None and (n <= GATED_MAX_ROWS or self.w_gu is None):
+            if normed:
+                ok = takes_prepared_norm(rt, n, self.width) if x.prepared else (can_fuse(rt, n) and self.width % 8 == 0)
+                if not ok:
+                    x, normed = x.materialize(), False
+            if normed and x.prepared:
+                ops.gated_linear_bf16_form(x.xn, self.p_gu, self.b_gu, act, self.alpha, self.limit, self.shift,
+                                           norm_eps=x.eps, ssq_in=x.ssq)
+            elif normed:
+                ops.gated_linear_bf16_form(x.h, self.p_gu, self.b_gu, act, self.alpha, self.limit, self.shift,
+                                           norm_gain=x.gain, norm_eps=x.eps)
+            else:
+                ops.gated_linear_bf16_form(x, self.p_gu, self.b_gu, act, self.alpha, self.limit, self.shift)
+        else:
+            gu = linear(rt, x, self.w_gu, self.b_gu, "mlp.gu", bias_lowp=self.b_gu_lowp)
+            ops.gated_act(gu, act, self.alpha, self.limit, self.shift)
+        return linear(rt, act, self.w_down, self.b_down, "mlp.down", bias_lowp=self.b_down_lowp, packed=self.p_down,
+                      residual=residual, hand_on=hand_on)
+
     def forward(self, x, ctx=None, residual: Optional[torch.Tensor] = None, hand_on=None):
         rt = self.rt
         n = x.shape[0]
         act = rt.buffer("mlp.act", (n, self.inter), rt.dtype)
         if not self.plain_silu or self.b_gu is not None:
-            # another form of the gate, or biases: the product (which takes the norm in front of it where it can), the
-            # gate as a kernel of its own, the down product
-            gu = linear(rt, x, self.w_gu, self.b_gu, "mlp.gu", bias_lowp=self.b_gu_lowp, packed=self.p_gu_plain)
-            ops.gated_act(gu, act, self.alpha, self.limit, self.shift)
-            return linear(rt, act, self.w_down, self.b_down, "mlp.down", bias_lowp=self.b_down_lowp, packed=self.p_down,
-                          residual=residual, hand_on=hand_on)
+            return self._forward_formed(x, act, residual, hand_on)
         normed = isinstance(x, NormedInput)
         if normed:
             ok = (takes_prepared_norm(rt, n, self.width) and self.p_gu is not None) if x.prepared else \

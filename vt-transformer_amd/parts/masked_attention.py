@@ -38,7 +38,7 @@ import torch
 from ..config.base import PartSpec
 from ..kernels import ops
 from .base import MIXERS, POSITIONS, CacheNeed, PageTensor, Part, Runtime, StateNeed, TensorDecl
-from .linear import linear
+from .linear import can_add_residual, linear
 
 
 TILE_ROWS = 16
@@ -73,7 +73,7 @@ class MaskedAttention(Part):
                  scale: Optional[float] = None, softcap: float = 0.0, window: int = 0, chunk: int = 0,
                  unit_rms_eps: Optional[float] = None, head_gate: bool = False, shared: Optional[dict] = None,
                  names: Optional[Dict[str, str]] = None, sink: bool = False, distance_slopes: Optional[float] = None,
-                 q_temp: Optional[Dict[str, float]] = None, value_mix: Optional[str] = None):
+                 q_temp: Optional[Dict[str, float]] = None, value_mix: Optional[str] = None, fuse_norms: bool = False):
         """key_dim / value_dim: sizes of a head's queries and keys / of its values (default: the same);
         position: a rotary encoding whose `dim` may be smaller than key_dim (the rest of a head passes unchanged);
         unit_rms_eps: queries and keys are divided by their root mean square per head after the rotation, with
@@ -82,7 +82,10 @@ class MaskedAttention(Part):
         k_bias, v_bias; sink: one learned number per head whose exponential joins the softmax's denominator;
         distance_slopes: s > 0 takes 2^(-s (h + 1) / H) times the distance off head h's scores; q_temp {coef, every}:
         the queries' factor by position; value_mix: "source" (this layer's values are what later layers mix in),
-        "mix" (this layer keeps (1 - lambda) v + lambda v_source, lambda its tensor `vmix`) or None."""
+        "mix" (this layer keeps (1 - lambda) v + lambda v_source, lambda its tensor `vmix`) or None; fuse_norms: with
+        few rows in bfloat16 the input product applies the norm in front of the mixer and the output product adds to
+        the residual stream and prepares the norm behind (as `PagedAttention` does; it rounds the stream times the
+        norm's gains to 16 bits before the division by the root instead of after it)."""
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
         self.rt, self.width = rt, int(width)
@@ -109,6 +112,8 @@ class MaskedAttention(Part):
         if value_mix not in (None, "source", "mix"):
             raise ValueError(f"value_mix {value_mix!r} ('source', 'mix' or None)")
         self.value_mix = value_mix
+        # what the block asks for (parts/block.py)
+        self.takes_normed_input = self.hands_norm_on = bool(fuse_norms)
         n = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight", "g": "g_proj.weight",
              "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "sink": "sink", "vmix": "vmix"}
         n.update(names or {})
@@ -195,7 +200,11 @@ class MaskedAttention(Part):
         self.p_in, self.p_o = rt.pack(self.w_in), rt.pack(self.w_o)
         self.w_in, self.w_o = rt.row_major(self.w_in, self.p_in), rt.row_major(self.w_o, self.p_o)
 
-    def forward(self, x, ctx, cache, state=None):
+    def adds_residual(self, rows: int) -> bool:
+        """Whether the output product adds to the residual stream itself at this many rows."""
+        return self.takes_normed_input and can_add_residual(self.rt, rows, self.width, self.nh * self.dv)
+
+    def forward(self, x, ctx, cache, state=None, residual: Optional[torch.Tensor] = None, hand_on=None):
         rt, nh, nkv, d, dv = self.rt, self.nh, self.nkv, self.d, self.dv
         n = x.shape[0]
         if not cache.writes:
@@ -215,9 +224,9 @@ class MaskedAttention(Part):
                                       nh, nkv, d, dv, self.scale, self.softcap, self.window, self.chunk,
                                       gate=y if self.head_gate else None, gate_column=self._gate_column,
                                       sink=self.sink, slopes=self.slopes)
-            return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o)
+            return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o, residual=residual, hand_on=hand_on)
         ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
                              dv, self.scale, self.softcap, self.window, self.chunk,
                              gate=y if self.head_gate else None, gate_column=self._gate_column,
                              sink=self.sink, slopes=self.slopes)
-        return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o)
+        return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o, residual=residual, hand_on=hand_on)
