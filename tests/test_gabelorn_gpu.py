@@ -213,9 +213,17 @@ def test_one_key_far_back_against_a_sink_and_slopes(dtype, matrix):
             out = torch.empty(b - a, nh * dv, dtype=dtype, device=DEV)
             ops.qk_prepare(yy, None, None, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, kvh,
                            d, dv, None)
-            if matrix and b - a > 1:        # (the mixer sends steps of single tokens to the other kernel)
+            if matrix and b - a > 1:
                 ops.attention_masked_mfma(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table,
                                           ctx.extra[TILES_KEY], out, nh, kvh, d, dv, 1.0, sink=sink, slopes=slopes)
+            elif matrix:                    # single tokens: the kernel whose rows are heads and whose keys are dealt out
+                for splits in (1, 3):
+                    part = torch.empty(ops.attention_masked_decode_scratch(1, nh, kvh, dv, splits), device=DEV)
+                    ops.attention_masked_decode(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table,
+                                                out, part, splits, nh, kvh, d, dv, 1.0, sink=sink, slopes=slopes)
+                    if splits == 1:
+                        first = out.clone()
+                assert float((out.float() - first.float()).abs().max()) < 0.3       # (however the keys are dealt out)
             else:
                 ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, kvh,
                                      d, dv, 1.0, sink=sink, slopes=slopes)

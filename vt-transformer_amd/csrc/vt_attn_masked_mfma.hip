@@ -433,6 +433,227 @@ __global__ __launch_bounds__(256) void attn_masked_mfma_shared_kernel(MfmaArgs a
     }
 }
 
+// ---------------------------------------------------------------------------
+// Steps of single tokens (decoding).  The 16 rows of the matrix products are not tokens but the query heads that share
+// a key/value head, all of one token: one read of a key serves the whole group, which for a mixer whose heads all read
+// one cache is every head.  The keys of a token are dealt out in turns of 32 to P = 4 x splits waves (turn i to wave
+// i mod P), each wave keeps its own running maximum, sum and weighted values and leaves them in `part`; a second
+// launch merges the P parts of every head, adds the sink to the denominator, applies the gate and writes the output.
+// The grid depends on the number of tokens and on `splits` alone, the keys' range is read from device memory: a step
+// can be recorded once and replayed.
+//   part: [token][group tile][P][16 rows][DV + 4] floats: weighted values, then maximum and sum (base 2)
+// ---------------------------------------------------------------------------
+struct DecodeArgs {
+    const bf16_t* q;        // [n][H][D]
+    const bf16_t* k_pages;
+    const bf16_t* v_pages;
+    const int* positions;
+    const int* tok_entry;
+    const int* block_table;
+    const float* sink;
+    const float* slopes;
+    const void* gate;
+    float* part;
+    bf16_t* out;            // [n][H][DV]
+    long long ldg;
+    int n, H, G, HT, P, page_size, max_blocks, num_pages, window, chunk, gate_f32;
+    float scale, cap;
+};
+#define DEC_ROW (VT_VALUE_DIM + 4)
+
+__global__ __launch_bounds__(256) void attn_masked_decode_kernel(DecodeArgs a) {
+    constexpr int D = VT_KEY_DIM, DV = VT_VALUE_DIM, NK = D / 16, NV = DV / 16;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, grp = lane >> 4;
+    const int p = blockIdx.x * 4 + wave, tile = blockIdx.y, t = blockIdx.z;
+    const int group = a.H / a.G;
+    const int kvh = tile / a.HT, ht = tile % a.HT;
+    const int rows = min(16, group - ht * 16);
+    const bool row_ok = r < rows;
+    const int h = kvh * group + ht * 16 + (row_ok ? r : 0);
+    const int pos = a.positions[t];
+    const int* bt = a.block_table + (size_t)a.tok_entry[t] * a.max_blocks;
+    const int ps = a.page_size;
+    int lo = a.chunk > 0 ? (pos / a.chunk) * a.chunk : 0;
+    if (a.window > 0) lo = max(lo, pos - a.window + 1);
+    const int kt0 = (lo / 16) * 16;
+    const int turns = (pos - kt0) / 32 + 1;
+
+    vt_lowp4_t qf[NK];
+    {
+        const bf16_t* qr = a.q + ((size_t)t * a.H + h) * D + grp * 4;
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) {
+            qf[kk] = load4(qr + kk * 16);
+            if (!row_ok) qf[kk] = (vt_lowp4_t){0, 0, 0, 0};
+        }
+    }
+    f32x4 acc[NV];
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[v] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const float nan = __int_as_float(0x7fc00000);
+    const float LOG2E = 1.4426950408889634f;
+    const float c1 = a.cap > 0.f ? a.scale * 2.0f * LOG2E / a.cap : a.scale * LOG2E;
+    const float c2 = a.cap * LOG2E;
+    const float slope2 = a.slopes ? a.slopes[h] * LOG2E : 0.f;
+
+    for (int turn = p; turn < turns; turn += a.P) {
+        const int kt = kt0 + turn * 32;
+        vt_lowp4_t kf[2][NK], vf[2][NV];
+        bool ok[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int k0 = kt + 16 * u;
+            const int blk = k0 / ps;
+            int pg = blk < a.max_blocks ? bt[blk] : -1;
+            ok[u] = pg >= 0 && pg < a.num_pages;
+            pg = ok[u] ? pg : 0;
+            const int slot0 = k0 % ps;
+            const bf16_t* kp = a.k_pages + (((size_t)pg * a.G + kvh) * ps + slot0 + r) * D + grp * 4;
+            const bf16_t* vp = a.v_pages + (((size_t)pg * a.G + kvh) * DV + r) * ps + slot0 + grp * 4;
+#pragma unroll
+            for (int kk = 0; kk < NK; ++kk) kf[u][kk] = load4(kp + kk * 16);
+#pragma unroll
+            for (int v = 0; v < NV; ++v) vf[u][v] = load4(vp + (size_t)v * 16 * ps);
+        }
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NK; ++kk) {
+            s0 = VT_MFMA_16X16X16(kf[0][kk], qf[kk], s0);
+            s1 = VT_MFMA_16X16X16(kf[1][kk], qf[kk], s1);
+        }
+        float sc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float x = (i < 4 ? s0[i] : s1[i - 4]) * c1;
+            if (a.cap > 0.f) {
+                const float e = __builtin_amdgcn_exp2f(x);
+                sc[i] = fmaf(-2.0f * c2, __builtin_amdgcn_rcpf(1.0f + e), c2);
+            } else {
+                sc[i] = x;
+            }
+            const int j = kt + (i < 4 ? 0 : 16) + grp * 4 + (i & 3);
+            if (a.slopes) sc[i] -= slope2 * (float)(pos - j);
+            const bool seen = row_ok && j <= pos && j >= lo;
+            // (a missing page must show, not pass as a masked key)
+            sc[i] = seen ? (ok[i >> 2] ? sc[i] : nan) : -INFINITY;
+        }
+        float mt = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m, mt);
+        const float mref = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+        float pr[8], psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pr[i] = __builtin_amdgcn_exp2f(sc[i] - mref);
+            psum += pr[i];
+        }
+        l = l * alpha + psum;
+        m = m_new;
+        struct U2 { unsigned a, b; };
+        const U2 pk0 = {vt_pack2(pr[0], pr[1]), vt_pack2(pr[2], pr[3])}, pk1 = {vt_pack2(pr[4], pr[5]), vt_pack2(pr[6], pr[7])};
+        const vt_lowp4_t pf0 = __builtin_bit_cast(vt_lowp4_t, pk0), pf1 = __builtin_bit_cast(vt_lowp4_t, pk1);
+#pragma unroll
+        for (int v = 0; v < NV; ++v) {
+            acc[v] *= alpha;
+            acc[v] = VT_MFMA_16X16X16(vf[0][v], pf0, acc[v]);
+            acc[v] = VT_MFMA_16X16X16(vf[1][v], pf1, acc[v]);
+        }
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!row_ok) return;
+    float* dst = a.part + ((((size_t)t * a.G * a.HT + tile) * a.P + p) * 16 + r) * DEC_ROW;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) *(float4*)(dst + v * 16 + grp * 4) = make_float4(acc[v][0], acc[v][1], acc[v][2], acc[v][3]);
+    if (grp == 0) {
+        dst[DV] = m;
+        dst[DV + 1] = l;
+    }
+}
+
+__global__ __launch_bounds__(64) void attn_masked_decode_merge_kernel(DecodeArgs a) {
+    constexpr int DV = VT_VALUE_DIM;
+    const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+    const int group = a.H / a.G;
+    const int kvh = h / group, within = h % group;
+    const int tile = kvh * a.HT + within / 16, r = within % 16;
+    const float* base = a.part + ((((size_t)t * a.G * a.HT + tile) * a.P) * 16 + r) * DEC_ROW;
+    const size_t step = (size_t)16 * DEC_ROW;
+    const float LOG2E = 1.4426950408889634f;
+    float m_all = -INFINITY;
+    for (int p = 0; p < a.P; ++p) m_all = fmaxf(m_all, base[p * step + DV]);
+    float keep = 1.f, extra = 0.f;
+    if (a.sink) {
+        // the sink is one more score with no value behind it
+        const float sk = a.sink[h] * LOG2E;
+        const float top = fmaxf(m_all, sk);
+        extra = __builtin_amdgcn_exp2f(sk - top);
+        m_all = top;
+    }
+    float l = extra;
+    for (int p = 0; p < a.P; ++p) {
+        const float mp = base[p * step + DV];
+        if (mp != -INFINITY) l += base[p * step + DV + 1] * __builtin_amdgcn_exp2f(mp - m_all);
+    }
+    float gate = 1.f;
+    if (a.gate) {
+        const size_t gi = (size_t)t * a.ldg + h;
+        const float z = a.gate_f32 ? ((const float*)a.gate)[gi] : bf16_to_f32(((const bf16_t*)a.gate)[gi]);
+        gate = 1.0f / (1.0f + expf(-z));
+    }
+    const float f = keep * gate / l;
+    bf16_t* o = a.out + ((size_t)t * a.H + h) * DV;
+    for (int d = lane; d < DV; d += 64) {
+        float sum = 0.f;
+        for (int p = 0; p < a.P; ++p) {
+            const float mp = base[p * step + DV];
+            if (mp != -INFINITY) sum += base[p * step + d] * __builtin_amdgcn_exp2f(mp - m_all);
+        }
+        o[d] = f32_to_bf16(sum * f);
+    }
+}
+
+extern "C" int vt_attn_masked_decode(const void* q, const void* k_pages, const void* v_pages, const int* positions,
+                                     const int* tok_entry, const int* block_table, const void* gate, int gate_dtype,
+                                     long long ldg, void* out, float* part, long long part_floats, int splits, int n,
+                                     int H, int G, int D, int Dv, int page_size, int max_blocks, int num_pages, int window,
+                                     int chunk, float scale, float cap, const float* sink, const float* slopes,
+                                     hipStream_t stream) {
+    VT_REQUIRE(D == VT_KEY_DIM && Dv == VT_VALUE_DIM, "vt_attn_masked_decode: built for heads of %d/%d, called with %d/%d",
+               VT_KEY_DIM, VT_VALUE_DIM, D, Dv);
+    VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked_decode: bad heads %d/%d", H, G);
+    VT_REQUIRE(page_size > 0 && page_size % 16 == 0 && max_blocks > 0 && num_pages > 0,
+               "vt_attn_masked_decode: pages of %d keys (a multiple of 16)", page_size);
+    VT_REQUIRE(window >= 0 && chunk >= 0 && cap >= 0.f, "vt_attn_masked_decode: bad mask or cap");
+    VT_REQUIRE(splits >= 1 && splits <= 64, "vt_attn_masked_decode: %d splits (1 to 64)", splits);
+    VT_REQUIRE(!gate || gate_dtype == VT_F32 || gate_dtype == VT_BF16, "vt_attn_masked_decode: gate dtype %d", gate_dtype);
+    if (n == 0) return 0;
+    const int HT = (H / G + 15) / 16;
+    VT_REQUIRE(n <= 65535 && G * HT <= 65535 && H <= 65535, "vt_attn_masked_decode: too many tokens or heads");
+    const long long need = (long long)n * G * HT * 4 * splits * 16 * DEC_ROW;
+    VT_REQUIRE(part && part_floats >= need && (((uintptr_t)part) & 15) == 0,
+               "vt_attn_masked_decode: %lld floats of scratch memory, %lld needed (16-byte aligned)", part_floats, need);
+    DecodeArgs a;
+    a.q = (const bf16_t*)q; a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages; a.positions = positions;
+    a.tok_entry = tok_entry; a.block_table = block_table; a.sink = sink; a.slopes = slopes; a.gate = gate; a.part = part;
+    a.out = (bf16_t*)out; a.ldg = ldg; a.n = n; a.H = H; a.G = G; a.HT = HT; a.P = 4 * splits; a.page_size = page_size;
+    a.max_blocks = max_blocks; a.num_pages = num_pages; a.window = window; a.chunk = chunk; a.gate_f32 = gate_dtype == VT_F32;
+    a.scale = scale; a.cap = cap;
+    attn_masked_decode_kernel<<<dim3(splits, G * HT, n), 256, 0, stream>>>(a);
+    VT_CHECK_LAUNCH("vt_attn_masked_decode");
+    attn_masked_decode_merge_kernel<<<dim3(H, n), 64, 0, stream>>>(a);
+    VT_CHECK_LAUNCH("vt_attn_masked_decode(merge)");
+    return 0;
+}
+
+extern "C" long long vt_attn_masked_decode_scratch(int n, int H, int G, int splits) {
+    return (long long)n * G * ((H / G + 15) / 16) * 4 * splits * 16 * DEC_ROW;
+}
+
 extern "C" int vt_attn_masked_mfma_dims(int* key_dim, int* value_dim) {
     *key_dim = VT_KEY_DIM;
     *value_dim = VT_VALUE_DIM;

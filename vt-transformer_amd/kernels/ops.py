@@ -878,6 +878,58 @@ def attention_masked_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
     return out
 
 
+def attention_masked_decode_splits(n: int, n_heads: int, n_kv: int, max_len: int) -> int:
+    """Into how many blocks of four waves a decoding step's keys are dealt per (token, group of heads): enough to give
+    every compute unit a few waves, no more than there are turns of 32 keys in the longest sequence.  It depends on
+    the number of tokens and the engine's limits alone, so that a recorded step can be replayed."""
+    tiles = max(1, n) * n_kv * (-(-(n_heads // n_kv) // 16))
+    return int(max(1, min(-(-512 // tiles), max(1, max_len // 128), 16)))
+
+
+def attention_masked_decode(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, positions: torch.Tensor,
+                            tok_entry: torch.Tensor, block_table: torch.Tensor, out: torch.Tensor, part: torch.Tensor,
+                            splits: int, n_heads: int, n_kv: int, key_dim: int, value_dim: int, scale: float,
+                            cap: float = 0.0, window: int = 0, chunk: int = 0, gate: Optional[torch.Tensor] = None,
+                            gate_column: int = 0, sink: Optional[torch.Tensor] = None,
+                            slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """attention_masked for steps of single tokens in the 16-bit types on the matrix cores: the rows of a product are
+    the query heads that share a key/value head.  part: float32 scratch of attention_masked_decode_scratch floats."""
+    n = q.shape[0]
+    num_pages, kvh, page_size, d = k_pages.shape
+    dt = _lowp(q, "attention_masked_decode.q")
+    if not attention_masked_mfma_takes(key_dim, value_dim, page_size):
+        raise KernelError(f"attention_masked_decode: heads of {key_dim}/{value_dim} and pages of {page_size} "
+                          f"(multiples of 16 up to 256)")
+    _chk(q, "attention_masked_decode.q", dt, (n, n_heads * key_dim))
+    _chk(k_pages, "attention_masked_decode.k_pages", dt, (num_pages, n_kv, page_size, key_dim))
+    _chk(v_pages, "attention_masked_decode.v_pages", dt, (num_pages, n_kv, value_dim, page_size))
+    _chk(out, "attention_masked_decode.out", dt, (n, n_heads * value_dim))
+    _chk(positions, "attention_masked_decode.positions", torch.int32, (n,))
+    _chk(tok_entry, "attention_masked_decode.tok_entry", torch.int32, (n,))
+    _chk(block_table, "attention_masked_decode.block_table", torch.int32)
+    _chk(part, "attention_masked_decode.part", torch.float32)
+    gptr, gcode, ldg = ctypes.c_void_p(0), F32, 0
+    if gate is not None:
+        _chk(gate, "attention_masked_decode.gate")
+        if gate.dim() != 2 or gate.shape[0] != n or gate.shape[1] < gate_column + n_heads:
+            raise KernelError(f"attention_masked_decode.gate: shape {tuple(gate.shape)} has no {n_heads} columns from {gate_column}")
+        gptr = ctypes.c_void_p(gate.data_ptr() + gate_column * gate.element_size())
+        gcode, ldg = _code(gate), gate.stride(0)
+    _per_head(sink, "attention_masked_decode.sink", n_heads)
+    _per_head(slopes, "attention_masked_decode.slopes", n_heads)
+    _run(load_lib("vt_attn_masked_mfma", (key_dim, value_dim), half=_half(q, gate)), "vt_attn_masked_decode", _ptr(q),
+         _ptr(k_pages), _ptr(v_pages), _ptr(positions), _ptr(tok_entry), _ptr(block_table), gptr, _i(gcode),
+         ctypes.c_longlong(ldg), _ptr(out), _ptr(part), ctypes.c_longlong(part.numel()), _i(splits), _i(n), _i(n_heads),
+         _i(n_kv), _i(key_dim), _i(value_dim), _i(page_size), _i(block_table.shape[1]), _i(num_pages), _i(window), _i(chunk),
+         _f(scale), _f(cap), _ptr(sink), _ptr(slopes), _stream())
+    return out
+
+
+def attention_masked_decode_scratch(n: int, n_heads: int, n_kv: int, value_dim: int, splits: int) -> int:
+    """Floats of scratch memory that attention_masked_decode needs."""
+    return n * n_kv * (-(-(n_heads // n_kv) // 16)) * 4 * splits * 16 * (value_dim + 4)
+
+
 # ---------------------------------------------------------------------------
 # attention over a low-rank cache (vt_latent.hip): what stands around the masked attention kernels
 HEAD_LINEAR_MAX_IN = 8192

@@ -30,7 +30,7 @@ from ..config.base import PartSpec
 from ..kernels import ops
 from .base import MIXERS, POSITIONS, CacheNeed, PageTensor, Part, Runtime, StateNeed, TensorDecl
 from .linear import can_add_residual, linear
-from .masked_attention import TILES_KEY, plan_tiles
+from .masked_attention import plan_tiles, run_masked_attention
 
 
 @MIXERS.register("latent_attention")
@@ -148,13 +148,7 @@ class LatentAttention(Part):
         # the unrotated query parts through W_uk^T, into the query rows in front of the rotated parts
         ops.head_linear(y, 0, dn + dr, self.w_uk, True, q, 0, dk, nh, dn, rank)
         mixed = rt.buffer("lattn.mixed", (n, nh * rank), rt.dtype)
-        tiles = ctx.extra.get(TILES_KEY) if self._matrix_cores() and not ctx.single_token else None
-        if tiles is not None and cache["k"].shape[2] % 16 == 0:
-            ops.attention_masked_mfma(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, tiles,
-                                      mixed, nh, 1, dk, rank, self.scale, 0.0, self.window, 0, sink=self.sink)
-        else:
-            ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, mixed, nh, 1,
-                                 dk, rank, self.scale, 0.0, self.window, 0, sink=self.sink)
+        run_masked_attention(rt, ctx, cache, q, mixed, nh, 1, dk, rank, self.scale, window=self.window, sink=self.sink)
         # the heads' mixed low-rank vectors through W_uv, times the gate
         out = rt.buffer("lattn.out", (n, nh * dv), rt.dtype)
         ops.head_linear(mixed, 0, rank, self.w_uv, False, out, 0, dv, nh, rank, dv,

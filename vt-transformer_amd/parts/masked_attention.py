@@ -59,6 +59,29 @@ def plan_tiles(ctx) -> Optional[Dict[tuple, np.ndarray]]:
     return {TILES_KEY: np.asarray(tiles, dtype=np.int32).reshape(-1)}
 
 
+def run_masked_attention(rt: Runtime, ctx, cache, q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, d: int, dv: int,
+                         scale: float, softcap: float = 0.0, window: int = 0, chunk: int = 0, gate=None,
+                         gate_column: int = 0, sink=None, slopes=None) -> torch.Tensor:
+    """The attention itself over a layer's pages, by the kernel that suits the step: in the 16-bit types with heads
+    in multiples of 16, steps of single tokens go to the matrix-core kernel whose rows are the heads of a key/value
+    group and whose keys are dealt out to many waves, steps with portions of prompts to the one whose rows are tokens
+    (tiles planned by `plan_tiles`); everything else, and float32 always, to the kernel with a block per (token, head)."""
+    cores = rt.lowp and ops.attention_masked_mfma_takes(d, dv, cache["k"].shape[2])
+    kw = dict(gate=gate, gate_column=gate_column, sink=sink, slopes=slopes)
+    if cores and ctx.single_token:
+        n = q.shape[0]
+        splits = ops.attention_masked_decode_splits(n, nh, nkv, ctx.n_positions)
+        part = rt.buffer("mattn.decode_parts", (ops.attention_masked_decode_scratch(n, nh, nkv, dv, splits),), torch.float32)
+        return ops.attention_masked_decode(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out,
+                                           part, splits, nh, nkv, d, dv, scale, softcap, window, chunk, **kw)
+    tiles = ctx.extra.get(TILES_KEY) if cores and not ctx.single_token else None
+    if tiles is not None:
+        return ops.attention_masked_mfma(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, tiles,
+                                         out, nh, nkv, d, dv, scale, softcap, window, chunk, **kw)
+    return ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv,
+                                d, dv, scale, softcap, window, chunk, **kw)
+
+
 def head_slopes(n_heads: int, steepness: float) -> np.ndarray:
     """slope_h = 2^(-steepness (h + 1) / H), float32."""
     return np.power(2.0, -float(steepness) * (np.arange(n_heads, dtype=np.float64) + 1.0) / n_heads).astype(np.float32)
@@ -218,15 +241,7 @@ class MaskedAttention(Part):
         ops.qk_prepare(y, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, nkv,
                        d, dv, self.unit_rms_eps, q_temp=self.q_temp, v_first=v_first, v_lambda=self.v_lambda)
         out = rt.buffer("mattn.out", (n, nh * dv), rt.dtype)
-        tiles = ctx.extra.get(TILES_KEY) if self._matrix_cores() and not ctx.single_token else None
-        if tiles is not None and cache["k"].shape[2] % 16 == 0:
-            ops.attention_masked_mfma(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, tiles, out,
-                                      nh, nkv, d, dv, self.scale, self.softcap, self.window, self.chunk,
-                                      gate=y if self.head_gate else None, gate_column=self._gate_column,
-                                      sink=self.sink, slopes=self.slopes)
-            return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o, residual=residual, hand_on=hand_on)
-        ops.attention_masked(q, cache["k"], cache["v"], ctx.positions, ctx.tok_entry, cache.block_table, out, nh, nkv, d,
-                             dv, self.scale, self.softcap, self.window, self.chunk,
-                             gate=y if self.head_gate else None, gate_column=self._gate_column,
-                             sink=self.sink, slopes=self.slopes)
+        run_masked_attention(rt, ctx, cache, q, out, nh, nkv, d, dv, self.scale, self.softcap, self.window, self.chunk,
+                             gate=y if self.head_gate else None, gate_column=self._gate_column, sink=self.sink,
+                             slopes=self.slopes)
         return linear(rt, out, self.w_o, None, "mattn.o", packed=self.p_o, residual=residual, hand_on=hand_on)
