@@ -284,6 +284,34 @@ def test_latent_window_edges_at_a_page_border(dtype, nh):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,heads,n_in,n_out,transposed,gated", [
+    (1, 3, 20, 24, False, True), (9, 8, 128, 48, False, False), (70, 2, 16, 100, True, True), (33, 5, 44, 12, True, False),
+    (200, 4, 64, 64, False, True),
+])
+def test_per_head_products(dtype, n, heads, n_in, n_out, transposed, gated):
+    """One small matrix per head, from and into columns of wider rows, in either orientation, with and without the gate;
+    float32 inputs to 16-bit results as well (what a few-row product hands on)."""
+    from vt_transformer_amd.kernels import ops
+    g = torch.Generator().manual_seed(n + heads)
+    x_cols, y_cols, x_head, y_head = 8 + heads * (n_in + 4), 4 + heads * (n_out + 8), n_in + 4, n_out + 8
+    w = (torch.randn(heads, n_out, n_in, generator=g) / n_in ** 0.5).to(torch.bfloat16).float()
+    gate = torch.randn(n, 12 + heads * n_out, generator=g)
+    for x_dtype in ({torch.float32, dtype}):
+        x = torch.randn(n, x_cols, generator=g).to(x_dtype)
+        y = torch.zeros(n, y_cols, dtype=dtype, device=DEV)
+        wd = (w.transpose(1, 2).contiguous() if transposed else w).reshape(-1, n_out if transposed else n_in).to(dtype).to(DEV)
+        ops.head_linear(x.to(DEV), 8, x_head, wd, transposed, y, 4, y_head, heads, n_in, n_out,
+                        gate=gate.to(x_dtype).to(DEV) if gated else None, gate_column=12)
+        xs = x.double()[:, 8:8 + heads * x_head].reshape(n, heads, x_head)[:, :, :n_in]
+        ref = torch.einsum("hoi,nhi->nho", w.double(), xs)
+        if gated:
+            ref = ref * torch.sigmoid(gate.to(x_dtype).double()[:, 12:12 + heads * n_out].reshape(n, heads, n_out))
+        got = y.float().cpu()[:, 4:4 + heads * y_head].reshape(n, heads, y_head)
+        assert rel(got[:, :, :n_out], ref) < PART_TOL[dtype]
+        assert float(got[:, :, n_out:].abs().max()) == 0.0 and float(y[:, :4].abs().max()) == 0.0    # nothing beside its columns
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("rows", [1, 5, 70, 300])
 def test_bounded_gated_feed_forward(dtype, rows):
     from vt_transformer_amd.parts import FEED_FORWARDS

@@ -575,18 +575,29 @@ __global__ __launch_bounds__(256) void attn_masked_decode_kernel(DecodeArgs a) {
     }
 }
 
-__global__ __launch_bounds__(64) void attn_masked_decode_merge_kernel(DecodeArgs a) {
+// A block per (token, head), a wave per 64 value elements: lane p takes part p's maximum and sum (P <= 64), the wave
+// finds the common maximum and every part's weight 2^(m_p - m), and each lane then adds up its value element over the
+// parts with those weights
+// (from LDS; an empty part weighs nothing), loads that do not wait for one another.
+#define MERGE_WAVES ((VT_VALUE_DIM + 63) / 64)
+__global__ __launch_bounds__(64 * MERGE_WAVES) void attn_masked_decode_merge_kernel(DecodeArgs a) {
     constexpr int DV = VT_VALUE_DIM;
-    const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+    __shared__ float ws_all[MERGE_WAVES][64];
+    float* ws = ws_all[threadIdx.x >> 6];       // (every wave works the weights out for itself: no barrier)
+    const int h = blockIdx.x, t = blockIdx.y, lane = threadIdx.x & 63;
     const int group = a.H / a.G;
     const int kvh = h / group, within = h % group;
     const int tile = kvh * a.HT + within / 16, r = within % 16;
     const float* base = a.part + ((((size_t)t * a.G * a.HT + tile) * a.P) * 16 + r) * DEC_ROW;
     const size_t step = (size_t)16 * DEC_ROW;
     const float LOG2E = 1.4426950408889634f;
-    float m_all = -INFINITY;
-    for (int p = 0; p < a.P; ++p) m_all = fmaxf(m_all, base[p * step + DV]);
-    float keep = 1.f, extra = 0.f;
+    float mp = -INFINITY, lp = 0.f;
+    if (lane < a.P) {
+        mp = base[lane * step + DV];
+        lp = base[lane * step + DV + 1];
+    }
+    float m_all = wave_max(mp);
+    float extra = 0.f;
     if (a.sink) {
         // the sink is one more score with no value behind it
         const float sk = a.sink[h] * LOG2E;
@@ -594,25 +605,23 @@ __global__ __launch_bounds__(64) void attn_masked_decode_merge_kernel(DecodeArgs
         extra = __builtin_amdgcn_exp2f(sk - top);
         m_all = top;
     }
-    float l = extra;
-    for (int p = 0; p < a.P; ++p) {
-        const float mp = base[p * step + DV];
-        if (mp != -INFINITY) l += base[p * step + DV + 1] * __builtin_amdgcn_exp2f(mp - m_all);
-    }
+    const float w = mp == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mp - m_all);
+    const float l = wave_sum(lp * w) + extra;
+    ws[lane] = w;
+    wave_lds_order();
     float gate = 1.f;
     if (a.gate) {
         const size_t gi = (size_t)t * a.ldg + h;
         const float z = a.gate_f32 ? ((const float*)a.gate)[gi] : bf16_to_f32(((const bf16_t*)a.gate)[gi]);
         gate = 1.0f / (1.0f + expf(-z));
     }
-    const float f = keep * gate / l;
+    const float f = gate / l;
     bf16_t* o = a.out + ((size_t)t * a.H + h) * DV;
-    for (int d = lane; d < DV; d += 64) {
+    const int d = threadIdx.x;                  // a wave per 64 value elements
+    if (d < DV) {
         float sum = 0.f;
-        for (int p = 0; p < a.P; ++p) {
-            const float mp = base[p * step + DV];
-            if (mp != -INFINITY) sum += base[p * step + d] * __builtin_amdgcn_exp2f(mp - m_all);
-        }
+#pragma unroll 8
+        for (int p = 0; p < a.P; ++p) sum = fmaf(base[p * step + d], ws[p], sum);
         o[d] = f32_to_bf16(sum * f);
     }
 }
@@ -645,7 +654,7 @@ extern "C" int vt_attn_masked_decode(const void* q, const void* k_pages, const v
     a.scale = scale; a.cap = cap;
     attn_masked_decode_kernel<<<dim3(splits, G * HT, n), 256, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_masked_decode");
-    attn_masked_decode_merge_kernel<<<dim3(H, n), 64, 0, stream>>>(a);
+    attn_masked_decode_merge_kernel<<<dim3(H, n), 64 * MERGE_WAVES, 0, stream>>>(a);
     VT_CHECK_LAUNCH("vt_attn_masked_decode(merge)");
     return 0;
 }

@@ -173,8 +173,16 @@ __global__ __launch_bounds__(256) void head_linear_kernel(HeadLinArgs a) {
 // The 16-bit product on the matrix cores: a wave takes 16 tokens, one head and 16 outputs; Y^T = W_h X^T
 // [16 outputs x 16 tokens] by v_mfma_f32_16x16x16 over the inputs.  A = W_h: a lane holds 4 consecutive inputs of its
 // output's row (W_h x) or gathers them from 4 rows (W_h^T x); B = X: 4 consecutive inputs of the lane's token.
-// Inputs beyond `in` and rows beyond n are zeros.  x and y are 16-bit; `in` is a multiple of 4.
+// Inputs beyond `in` and rows beyond n are zeros.  y is 16-bit, x 16-bit or float32 (rounded on its way in); `in` is a
+// multiple of 4.
 typedef __attribute__((ext_vector_type(4))) float hl_f32x4;
+__device__ __forceinline__ vt_lowp4_t load_x4(const bf16_t* p) { return *(const vt_lowp4_t*)p; }
+__device__ __forceinline__ vt_lowp4_t load_x4(const float* p) {
+    const float4 v = *(const float4*)p;
+    struct { unsigned a, b; } u = {vt_pack2(v.x, v.y), vt_pack2(v.z, v.w)};
+    return __builtin_bit_cast(vt_lowp4_t, u);
+}
+template <typename TX>
 __global__ __launch_bounds__(256) void head_linear_mfma_kernel(HeadLinArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, grp = lane >> 4;
@@ -185,7 +193,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(HeadLinArgs a) {
     const int ot = item % otiles, h = (item / otiles) % a.H, tt = item / (otiles * a.H);
     const int t = tt * 16 + r, o = ot * 16 + r;
     const bool t_ok = t < a.n, o_ok = o < a.out;
-    const bf16_t* x = (const bf16_t*)a.x + (size_t)(t_ok ? t : 0) * a.ldx + (size_t)h * a.x_head;
+    const TX* x = (const TX*)a.x + (size_t)(t_ok ? t : 0) * a.ldx + (size_t)h * a.x_head;
     const bf16_t* w = (const bf16_t*)a.w + (size_t)h * a.in * a.out;
     hl_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     const vt_lowp4_t zero = {0, 0, 0, 0};
@@ -193,7 +201,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(HeadLinArgs a) {
         const int k = k0 + grp * 4;
         const bool k_ok = k < a.in;                     // (in is a multiple of 4: a lane's four inputs are all in or all out)
         vt_lowp4_t xb = zero, wa = zero;
-        if (k_ok && t_ok) xb = *(const vt_lowp4_t*)(x + k);
+        if (k_ok && t_ok) xb = load_x4(x + k);
         if (k_ok && o_ok) {
             if (a.transposed) {
                 struct { bf16_t e[4]; } g;
@@ -231,11 +239,12 @@ extern "C" int vt_head_linear(const void* x, int x_dtype, long long ldx, int x_h
     a.x = x; a.w = w; a.gate = gate; a.y = y; a.ldx = ldx; a.ldy = ldy; a.ldg = ldg; a.x_head = x_head; a.y_head = y_head;
     a.n = n; a.H = H; a.in = in; a.out = out; a.transposed = transposed; a.gate_f32 = gate_dtype == VT_F32;
     if (matrix_cores) {
-        VT_REQUIRE(x_dtype == VT_BF16 && y_dtype == VT_BF16, "vt_head_linear: the matrix cores take 16-bit inputs");
-        VT_REQUIRE(in % 4 == 0 && ldx % 4 == 0 && x_head % 4 == 0 && ((uintptr_t)x & 7) == 0 && ((uintptr_t)w & 7) == 0,
-                   "vt_head_linear: the matrix cores take inputs in aligned groups of four");
+        VT_REQUIRE(y_dtype == VT_BF16, "vt_head_linear: the matrix cores give 16-bit results");
+        VT_REQUIRE(in % 4 == 0 && ldx % 4 == 0 && x_head % 4 == 0 && ((uintptr_t)x & (x_dtype == VT_F32 ? 15 : 7)) == 0 &&
+                   ((uintptr_t)w & 7) == 0, "vt_head_linear: the matrix cores take inputs in aligned groups of four");
         const long long items = (long long)((n + 15) / 16) * H * ((out + 15) / 16);
-        head_linear_mfma_kernel<<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(a);
+        if (x_dtype == VT_F32) head_linear_mfma_kernel<float><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(a);
+        else head_linear_mfma_kernel<bf16_t><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(a);
         VT_CHECK_LAUNCH("vt_head_linear");
         return 0;
     }

@@ -985,7 +985,7 @@ def head_linear(x: torch.Tensor, x_column: int, x_head: int, w: torch.Tensor, tr
     """One small matrix per head: y[t, y_column + h * y_head + o] = sum_i W_h[o, i] x[t, x_column + h * x_head + i]
     (w [H * n_out, n_in]), or with `transposed` sum_i W_h[i, o] x[...] (w [H * n_in, n_out]); times
     sigmoid(gate[t, gate_column + h * n_out + o]) if `gate` is given.  x and y are 2-d tensors whose rows are the
-    tokens'; float32 sums.  16-bit inputs go to the matrix cores."""
+    tokens'; float32 sums.  16-bit results come from the matrix cores (float32 inputs are rounded on their way in)."""
     n = x.shape[0]
     _chk(x, "head_linear.x")
     _chk(y, "head_linear.y")
@@ -1011,7 +1011,7 @@ def head_linear(x: torch.Tensor, x_column: int, x_head: int, w: torch.Tensor, tr
         gcode, ldg = _code(gate), gate.stride(0)
     xptr = ctypes.c_void_p(x.data_ptr() + x_column * x.element_size())
     yptr = ctypes.c_void_p(y.data_ptr() + y_column * y.element_size())
-    cores = (x.dtype in LOWP and n_in % 4 == 0 and x_head % 4 == 0 and x.stride(0) % 4 == 0 and x_column % 4 == 0)
+    cores = (y.dtype in LOWP and n_in % 4 == 0 and x_head % 4 == 0 and x.stride(0) % 4 == 0 and x_column % 4 == 0)
     _run(load_lib("vt_latent", half=_half(x, y, gate)), "vt_head_linear", xptr, _i(_code(x)), ctypes.c_longlong(x.stride(0)),
          _i(x_head), _ptr(w), gptr, _i(gcode), ctypes.c_longlong(ldg), yptr, _i(_code(y)), ctypes.c_longlong(y.stride(0)),
          _i(y_head), _i(n), _i(n_heads), _i(n_in), _i(n_out), _i(1 if transposed else 0), _i(1 if cores else 0), _stream())

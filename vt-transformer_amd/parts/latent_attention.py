@@ -121,7 +121,11 @@ class LatentAttention(Part):
         mats = [rt.place(get(nm[k]), "matrix") for k in (("q", "dkv", "g") if self.out_gate else ("q", "dkv"))]
         self.w_in = torch.cat(mats, dim=0).contiguous()
         self.w_o = rt.place(get(nm["o"]), "matrix")
-        self.w_uk, self.w_uv = rt.place(get(nm["uk"]), "matrix"), rt.place(get(nm["uv"]), "matrix")
+        # W_uk is only ever used transposed (queries go through it, not the cache): kept as [H][rank][plain_dim], so
+        # that both per-head products read a matrix row by row
+        w_uk = rt.place(get(nm["uk"]), "matrix")
+        self.w_uk = w_uk.view(self.nh, self.dn, self.rank).transpose(1, 2).contiguous().view(self.nh * self.rank, self.dn)
+        self.w_uv = rt.place(get(nm["uv"]), "matrix")
         self.norm_w = rt.place(get(nm["dkv_norm"]), "gain")
         if self.has_sink:
             self.sink = rt.place(get(nm["sink"]), "bias")
@@ -146,7 +150,7 @@ class LatentAttention(Part):
         ops.latent_prepare(y, 0, self._c_column, self.norm_w, self.eps, cos, sin, ctx.positions, ctx.tok_entry,
                            cache.block_table, q, cache["k"], cache["v"], nh, dn, dr, rank)
         # the unrotated query parts through W_uk^T, into the query rows in front of the rotated parts
-        ops.head_linear(y, 0, dn + dr, self.w_uk, True, q, 0, dk, nh, dn, rank)
+        ops.head_linear(y, 0, dn + dr, self.w_uk, False, q, 0, dk, nh, dn, rank)
         mixed = rt.buffer("lattn.mixed", (n, nh * rank), rt.dtype)
         run_masked_attention(rt, ctx, cache, q, mixed, nh, 1, dk, rank, self.scale, window=self.window, sink=self.sink)
         # the heads' mixed low-rank vectors through W_uv, times the gate
