@@ -286,7 +286,7 @@ def test_latent_window_edges_at_a_page_border(dtype, nh):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n,heads,n_in,n_out,transposed,gated", [
     (1, 3, 20, 24, False, True), (9, 8, 128, 48, False, False), (70, 2, 16, 100, True, True), (33, 5, 44, 12, True, False),
-    (200, 4, 64, 64, False, True),
+    (200, 4, 64, 64, False, True), (2100, 16, 128, 40, False, True), (1030, 32, 100, 48, False, False),   # (many tokens: 32 to a wave)
 ])
 def test_per_head_products(dtype, n, heads, n_in, n_out, transposed, gated):
     """One small matrix per head, from and into columns of wider rows, in either orientation, with and without the gate;

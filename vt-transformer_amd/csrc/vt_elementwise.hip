@@ -382,9 +382,46 @@ __global__ __launch_bounds__(256) void gated_act_vec_kernel(const TI* __restrict
                            bounded_gate(g.z, u.z, alpha, limit, shift), bounded_gate(g.w, u.w, alpha, limit, shift)));
     }
 }
+// 16-bit in and out, widths that are a multiple of 8: silu_mul_bf16x8_kernel's arrangement (a thread takes eight
+// columns in four rows, eight 16-byte loads asked for before any is used, marked non-temporal)
+__device__ __forceinline__ unsigned bounded_gate_pair(unsigned g, unsigned u, float alpha, float limit, float shift) {
+    return vt_pack2(bounded_gate(lowp_lo(g), lowp_lo(u), alpha, limit, shift), bounded_gate(lowp_hi(g), lowp_hi(u), alpha, limit, shift));
+}
+__global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
+                                                              int inter, int n, float alpha, float limit, float shift) {
+    typedef unsigned u32x4_t __attribute__((ext_vector_type(4)));
+    const int c = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (c >= inter) return;
+    const int t0 = blockIdx.y * 4;
+    u32x4_t g[4], u[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        if (t0 + k < n) {
+            const bf16_t* row = gu + (size_t)(t0 + k) * 2 * inter + c;
+            g[k] = __builtin_nontemporal_load((const u32x4_t*)row);
+            u[k] = __builtin_nontemporal_load((const u32x4_t*)(row + inter));
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        if (t0 + k < n) {
+            u32x4_t o;
+            o.x = bounded_gate_pair(g[k].x, u[k].x, alpha, limit, shift); o.y = bounded_gate_pair(g[k].y, u[k].y, alpha, limit, shift);
+            o.z = bounded_gate_pair(g[k].z, u[k].z, alpha, limit, shift); o.w = bounded_gate_pair(g[k].w, u[k].w, alpha, limit, shift);
+            *(u32x4_t*)(out + (size_t)(t0 + k) * inter + c) = o;
+        }
+    }
+}
 template <typename TI, typename TO>
 static void launch_gated_act(const void* gu, void* out, int n, int inter, float alpha, float limit, float shift,
                              hipStream_t stream) {
+    if constexpr (sizeof(TI) == 2 && sizeof(TO) == 2) {
+        if (inter % 8 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
+            const dim3 grid((inter / 8 + 255) / 256, (n + 3) / 4);
+            gated_act_bf16x8_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, inter, n, alpha, limit, shift);
+            return;
+        }
+    }
     if (inter % 4 == 0 && !((uintptr_t)gu & 15) && !((uintptr_t)out & 15)) {
         long long blocks = ((long long)(inter / 4) * n + 255) / 256;
         if (blocks > 16384) blocks = 16384;

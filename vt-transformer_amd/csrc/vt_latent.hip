@@ -224,6 +224,77 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(HeadLinArgs a) {
     }
 }
 
+// Many tokens: a wave takes 32 tokens and one head, keeps their inputs in registers (KS steps of 16: in <= 16 KS) and
+// goes through the head's output tiles, so that the tokens are read once and a row of W_h once per 32 tokens.
+// W_h as [out][in] only.
+template <typename TX, int KS>
+__global__ __launch_bounds__(256) void head_linear_mfma_rows_kernel(HeadLinArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, grp = lane >> 4;
+    const int item = blockIdx.x * 4 + wave;             // (pair of token tiles, head); heads fastest
+    const int tpairs = (a.n + 31) / 32;
+    if (item >= tpairs * a.H) return;
+    const int h = item % a.H, t0 = (item / a.H) * 32;
+    const vt_lowp4_t zero = {0, 0, 0, 0};
+    vt_lowp4_t xb[2][KS];
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+        const int t = t0 + 16 * u + r;
+        const TX* x = (const TX*)a.x + (size_t)(t < a.n ? t : 0) * a.ldx + (size_t)h * a.x_head;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            const int k = kk * 16 + grp * 4;
+            xb[u][kk] = (t < a.n && k < a.in) ? load_x4(x + k) : zero;
+        }
+    }
+    const bf16_t* w = (const bf16_t*)a.w + (size_t)h * a.in * a.out;
+    for (int ot = 0; ot * 16 < a.out; ++ot) {
+        const int o = ot * 16 + r;
+        vt_lowp4_t wa[KS];
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            const int k = kk * 16 + grp * 4;
+            wa[kk] = (o < a.out && k < a.in) ? *(const vt_lowp4_t*)(w + (size_t)o * a.in + k) : zero;
+        }
+        hl_f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            acc0 = VT_MFMA_16X16X16(wa[kk], xb[0][kk], acc0);
+            acc1 = VT_MFMA_16X16X16(wa[kk], xb[1][kk], acc1);
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int t = t0 + 16 * u + r;
+            if (t >= a.n) continue;
+            bf16_t* y = (bf16_t*)a.y + (size_t)t * a.ldy + (size_t)h * a.y_head;
+            const int oo = ot * 16 + grp * 4;
+            const hl_f32x4 acc = u ? acc1 : acc0;
+            if (oo + 3 < a.out && ((a.ldy | a.y_head) & 3) == 0 && (((uintptr_t)a.y) & 7) == 0) {
+                struct { unsigned lo, hi; } pk = {vt_pack2(gated(acc[0], a, t, h, oo), gated(acc[1], a, t, h, oo + 1)),
+                                                  vt_pack2(gated(acc[2], a, t, h, oo + 2), gated(acc[3], a, t, h, oo + 3))};
+                *(uint2*)(y + oo) = __builtin_bit_cast(uint2, pk);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    if (oo + e < a.out) y[oo + e] = f32_to_bf16(gated(acc[e], a, t, h, oo + e));
+            }
+        }
+    }
+}
+
+template <typename TX>
+static bool launch_head_rows(const HeadLinArgs& a, hipStream_t stream) {
+    // (worth it from a few hundred waves on; below that the kernel with a wave per output tile fills the GPU better)
+    const long long items = (long long)((a.n + 31) / 32) * a.H;
+    if (a.transposed || a.in > 256 || items < 512) return false;
+    const unsigned blocks = (unsigned)((items + 3) / 4);
+    if (a.in <= 64) head_linear_mfma_rows_kernel<TX, 4><<<blocks, 256, 0, stream>>>(a);
+    else if (a.in <= 128) head_linear_mfma_rows_kernel<TX, 8><<<blocks, 256, 0, stream>>>(a);
+    else if (a.in <= 192) head_linear_mfma_rows_kernel<TX, 12><<<blocks, 256, 0, stream>>>(a);
+    else head_linear_mfma_rows_kernel<TX, 16><<<blocks, 256, 0, stream>>>(a);
+    return true;
+}
+
 extern "C" int vt_head_linear(const void* x, int x_dtype, long long ldx, int x_head, const void* w, const void* gate,
                               int gate_dtype, long long ldg, void* y, int y_dtype, long long ldy, int y_head, int n,
                               int H, int in, int out, int transposed, int matrix_cores, hipStream_t stream) {
@@ -242,6 +313,10 @@ extern "C" int vt_head_linear(const void* x, int x_dtype, long long ldx, int x_h
         VT_REQUIRE(y_dtype == VT_BF16, "vt_head_linear: the matrix cores give 16-bit results");
         VT_REQUIRE(in % 4 == 0 && ldx % 4 == 0 && x_head % 4 == 0 && ((uintptr_t)x & (x_dtype == VT_F32 ? 15 : 7)) == 0 &&
                    ((uintptr_t)w & 7) == 0, "vt_head_linear: the matrix cores take inputs in aligned groups of four");
+        if (x_dtype == VT_F32 ? launch_head_rows<float>(a, stream) : launch_head_rows<bf16_t>(a, stream)) {
+            VT_CHECK_LAUNCH("vt_head_linear(rows)");
+            return 0;
+        }
         const long long items = (long long)((n + 15) / 16) * H * ((out + 15) / 16);
         if (x_dtype == VT_F32) head_linear_mfma_kernel<float><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(a);
         else head_linear_mfma_kernel<bf16_t><<<(unsigned)((items + 3) / 4), 256, 0, stream>>>(a);
