@@ -384,8 +384,17 @@ __global__ __launch_bounds__(256) void gated_act_vec_kernel(const TI* __restrict
 }
 // 16-bit in and out, widths that are a multiple of 8: silu_mul_bf16x8_kernel's arrangement (a thread takes eight
 // columns in four rows, eight 16-byte loads asked for before any is used, marked non-temporal)
+// (the division as one reciprocal instruction, 1 ulp, far below the 16-bit rounding of the result)
+__device__ __forceinline__ float bounded_gate_fast(float g, float u, float alpha, float limit, float shift) {
+    if (limit > 0.f) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+    }
+    return g * __builtin_amdgcn_rcpf(1.f + __expf(-alpha * g)) * (u + shift);
+}
 __device__ __forceinline__ unsigned bounded_gate_pair(unsigned g, unsigned u, float alpha, float limit, float shift) {
-    return vt_pack2(bounded_gate(lowp_lo(g), lowp_lo(u), alpha, limit, shift), bounded_gate(lowp_hi(g), lowp_hi(u), alpha, limit, shift));
+    return vt_pack2(bounded_gate_fast(lowp_lo(g), lowp_lo(u), alpha, limit, shift),
+                    bounded_gate_fast(lowp_hi(g), lowp_hi(u), alpha, limit, shift));
 }
 __global__ __launch_bounds__(256) void gated_act_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out,
                                                               int inter, int n, float alpha, float limit, float shift) {
