@@ -26,7 +26,7 @@ def test_configuration_becomes_parts():
     assert kinds == ["masked_attention", "latent_attention", "masked_attention", "masked_attention", "latent_attention",
                      "masked_attention"]
     # the first layer that mixes values is their source, the later ones mix, a layer that says no does neither
-    assert [ls.mixer.params.get("value_mix") for ls in spec.layers] == ["source", None, None, "mix", None, "mix"]
+    assert [ls.mixer.params.get("value_mix") for ls in spec.layers] == ["source", None, "off", "mix", None, "mix"]
     a = spec.layers[3].mixer.params
     assert (a["num_heads"], a["num_kv_heads"], a["key_dim"], a["value_dim"]) == (6, 2, 32, 48)
     assert a["q_temp"] == {"coef": 0.7, "every": 1} and a["distance_slopes"] == 8.0 and a["sink"] is True
@@ -54,7 +54,7 @@ def test_declared_tensors():
     assert t["l0.mix.q"].shape == (128, 96) and t["l0.mix.k"].shape == (64, 96) and t["l0.mix.v"].shape == (96, 96)
     assert t["l0.mix.o"].shape == (96, 4 * 48) and t["l0.mix.sink"].shape == (4,)
     assert t["l3.mix.vmix"].shape == () and not t["l3.mix.vmix"].optional and t["l0.mix.vmix"].optional
-    assert "l2.mix.vmix" not in t and "l2.norm2" not in t and "l2.mlp.gate" not in t
+    assert t["l2.mix.vmix"].optional and "l2.norm2" not in t and "l2.mlp.gate" not in t    # (tolerated, never read)
     assert t["l0.mlp.gate.b"].shape == (80,) and t["l0.mlp.down.b"].shape == (96,) and t["l0.mlp.up"].shape == (80, 96)
     assert not any(".b" == n[-2:] for n in t if ".mix." in n)        # no biases in the mixers
 
@@ -193,3 +193,26 @@ def test_plain_forward_shapes_and_cap():
     # causal: a longer sequence does not change earlier positions
     assert torch.allclose(pg.forward(cfg, w, [3, 1, 4, 1, 5])[:5], logits[:5], atol=1e-12)
     assert len(pg.greedy(cfg, w, [1, 2, 3], 3)) == 3
+
+
+def test_command_line_writes_a_random_model(tmp_path):
+    """`--write-random-model` with a Gabelorn config.json: the folder holds the configuration back and every tensor the
+    parts need."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from vt_transformer_amd.weights.safetensors_io import WeightStore
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg_path, out = tmp_path / "c.json", tmp_path / "m"
+    cfg_path.write_text(json.dumps(CFG_B))
+    r = subprocess.run([sys.executable, "-m", "vt_transformer_amd", "--write-random-model", str(out), "--config", str(cfg_path),
+                        "--seed", "9"], capture_output=True, text=True, env=dict(os.environ, PYTHONPATH=root), timeout=300)
+    assert r.returncode == 0, r.stderr
+    cfg = json.loads((out / "config.json").read_text())
+    assert cfg["architecture"] == "Gabelorn" and cfg["layers"] == CFG_B["layers"] and "logit_softcap" not in cfg
+    store = WeightStore(str(out))
+    names = set(store.names())
+    assert {"embed", "head", "final.norm", "l0.mix.dkv.norm", "l0.mix.uk", "l1.mix.sink", "l2.mix.g", "l1.mlp.down.b"} <= names
+    assert "l3.norm2" not in names and "l1.mix.vmix" not in names       # no feed-forward; the one mixing layer's number is not needed
+    store.close()

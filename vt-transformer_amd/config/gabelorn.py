@@ -187,7 +187,7 @@ class GabelornConfig(ModelConfig):
         layers = []
         seen_mixing = False
         for i, L in enumerate(self.layers):
-            value_mix = None
+            value_mix = "off" if L["type"] == "attention" else None
             if L["type"] == "attention" and L["mixer"].get("v_mix"):
                 value_mix = "mix" if seen_mixing else "source"
                 seen_mixing = True

@@ -204,11 +204,13 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
     for (int d = tid; d < D; d += KEYS) qs[d] = load_f32<TC>((const TC*)a.q, ((size_t)t * a.H + h) * D + d);
     __syncthreads();
 
-    const int Gv = KEYS / Dv;     // key groups for the weighted sum (Dv <= 256)
-    const int d_own = tid % Dv, g_own = tid / Dv;
+    const bool wide = Dv > KEYS;  // value heads wider than the block: a thread takes columns tid, tid + KEYS, ... (up to 4)
+    const int Gv = wide ? 1 : KEYS / Dv;     // key groups for the weighted sum
+    const int d_own = wide ? tid : tid % Dv, g_own = wide ? 0 : tid / Dv;
     const bool pv_active = g_own < Gv;
 
     float m = -INFINITY, l = 0.f, acc = 0.f;
+    float acc_w[3] = {0.f, 0.f, 0.f};        // columns tid + KEYS, tid + 2 KEYS, tid + 3 KEYS of a wide head
     for (int c0 = (lo / KEYS) * KEYS; c0 <= pos; c0 += KEYS) {
         const int j = c0 + tid;
         const bool valid = j >= lo && j <= pos;
@@ -246,6 +248,23 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
                 part = fmaf(sp[jj], load_f32<TC>(vp, (((size_t)pg * a.G + kvh) * Dv + d_own) * ps + (jk - blk * ps)), part);
             }
         }
+        if (wide) {
+#pragma unroll
+            for (int c = 1; c < 4; ++c) {
+                const int d = tid + c * KEYS;
+                if (d >= Dv) break;
+                float pw = 0.f;
+                for (int jj = 0; jj < KEYS; ++jj) {
+                    const int jk = c0 + jj;
+                    if (jk < lo || jk > pos) continue;
+                    const int blk = jk / ps;
+                    const int pg = bt[blk];
+                    if (pg < 0 || pg >= a.num_pages) continue;
+                    pw = fmaf(sp[jj], load_f32<TC>(vp, (((size_t)pg * a.G + kvh) * Dv + d) * ps + (jk - blk * ps)), pw);
+                }
+                acc_w[c - 1] = acc_w[c - 1] * alpha + pw;
+            }
+        }
         spart[tid] = part;
         __syncthreads();
         if (tid < Dv) {
@@ -263,6 +282,13 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
         const float keep = expf(m - m_all);
         l = l * keep + expf(sk - m_all);
         acc *= keep;
+#pragma unroll
+        for (int c = 0; c < 3; ++c) acc_w[c] *= keep;
+    }
+    float f = 1.0f / l;
+    if (a.gate) {
+        const float z = load_f32<TG>((const TG*)a.gate, (size_t)t * a.ldg + h);
+        f = (1.0f / (1.0f + expf(-z))) / l;
     }
     if (tid < Dv) {
         float o = acc / l;
@@ -272,6 +298,11 @@ __global__ __launch_bounds__(KEYS) void attn_masked_kernel(MaskedArgs a) {
         }
         store_f32<TC>((TC*)a.out, ((size_t)t * a.H + h) * Dv + tid, o);
     }
+    if (wide) {
+#pragma unroll
+        for (int c = 1; c < 4; ++c)
+            if (tid + c * KEYS < Dv) store_f32<TC>((TC*)a.out, ((size_t)t * a.H + h) * Dv + tid + c * KEYS, acc_w[c - 1] * f);
+    }
 }
 
 extern "C" int vt_attn_masked(const void* q, const void* k_pages, const void* v_pages, int dtype, const int* positions,
@@ -280,7 +311,7 @@ extern "C" int vt_attn_masked(const void* q, const void* k_pages, const void* v_
                               int max_blocks, int num_pages, int window, int chunk, float scale, float cap,
                               const float* sink, const float* slopes, hipStream_t stream) {
     VT_REQUIRE(n >= 0 && H > 0 && G > 0 && H % G == 0, "vt_attn_masked: bad heads %d/%d", H, G);
-    VT_REQUIRE(D > 0 && Dv > 0 && Dv <= 256, "vt_attn_masked: head sizes %d/%d (values up to 256)", D, Dv);
+    VT_REQUIRE(D > 0 && D <= 8192 && Dv > 0 && Dv <= 4 * KEYS, "vt_attn_masked: head sizes %d/%d (keys up to 8192, values up to %d)", D, Dv, 4 * KEYS);
     VT_REQUIRE(page_size > 0 && max_blocks > 0 && num_pages > 0, "vt_attn_masked: bad cache sizes");
     VT_REQUIRE(H <= 65535, "vt_attn_masked: too many heads (%d)", H);
     VT_REQUIRE(window >= 0 && chunk >= 0 && cap >= 0.f, "vt_attn_masked: bad mask or cap");

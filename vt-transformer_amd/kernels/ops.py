@@ -718,8 +718,9 @@ def attention_bf16_decode_fused(qkv: torch.Tensor, cos: Optional[torch.Tensor], 
 
 # ---------------------------------------------------------------------------
 # attention with separate key and value sizes, capped scores, chunk or window masks and head gates (vt_attn_masked.hip)
-MASKED_MAX_KEY_DIM = 256
-MASKED_MAX_VALUE_DIM = 256
+MASKED_MAX_KEY_DIM = 256        # what vt_qk_prepare takes
+MASKED_MAX_VALUE_DIM = 1024     # what vt_attn_masked takes (its keys: up to ATTN_MASKED_MAX_KEY_DIM); the matrix-core kernels 256
+ATTN_MASKED_MAX_KEY_DIM = 8192
 
 
 def qk_prepare(x: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,

@@ -53,9 +53,10 @@ class LatentAttention(Part):
         if min(self.nh, self.dn, self.dv, self.rank) <= 0 or self.dr < 0:
             raise ValueError("latent attention: heads and sizes must be positive")
         self.dk = self.rank + self.dr
-        if self.dk > ops.MASKED_MAX_KEY_DIM or self.rank > ops.MASKED_MAX_VALUE_DIM:
+        # (beyond 256 the matrix-core kernels do not take them: the kernel with a block per (token, head) does it all)
+        if self.dk > ops.ATTN_MASKED_MAX_KEY_DIM or self.rank > ops.MASKED_MAX_VALUE_DIM:
             raise ValueError(f"latent attention: rank {self.rank} + {self.dr} rotated elements: the attention kernels take keys "
-                             f"up to {ops.MASKED_MAX_KEY_DIM} and values up to {ops.MASKED_MAX_VALUE_DIM}")
+                             f"up to {ops.ATTN_MASKED_MAX_KEY_DIM} and values up to {ops.MASKED_MAX_VALUE_DIM}")
         self.eps = float(norm_eps)
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.dn + self.dr)
         self.window = int(window)

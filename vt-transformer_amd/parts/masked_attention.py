@@ -105,7 +105,9 @@ class MaskedAttention(Part):
         k_bias, v_bias; sink: one learned number per head whose exponential joins the softmax's denominator;
         distance_slopes: s > 0 takes 2^(-s (h + 1) / H) times the distance off head h's scores; q_temp {coef, every}:
         the queries' factor by position; value_mix: "source" (this layer's values are what later layers mix in),
-        "mix" (this layer keeps (1 - lambda) v + lambda v_source, lambda its tensor `vmix`) or None; fuse_norms: with
+        "mix" (this layer keeps (1 - lambda) v + lambda v_source, lambda its tensor `vmix`), "off" (neither, in a
+        model whose checkpoints may hold a `vmix` for such a layer all the same: it is tolerated and not read) or
+        None; fuse_norms: with
         few rows in bfloat16 the input product applies the norm in front of the mixer and the output product adds to
         the residual stream and prepares the norm behind (as `PagedAttention` does; it rounds the stream times the
         norm's gains to 16 bits before the division by the root instead of after it)."""
@@ -132,8 +134,8 @@ class MaskedAttention(Part):
             self.q_temp = (float(q_temp["coef"]), int(q_temp["every"]))
             if self.q_temp[1] <= 0:
                 raise ValueError(f"q_temp.every {self.q_temp[1]} must be positive")
-        if value_mix not in (None, "source", "mix"):
-            raise ValueError(f"value_mix {value_mix!r} ('source', 'mix' or None)")
+        if value_mix not in (None, "off", "source", "mix"):
+            raise ValueError(f"value_mix {value_mix!r} ('source', 'mix', 'off' or None)")
         self.value_mix = value_mix
         # what the block asks for (parts/block.py)
         self.takes_normed_input = self.hands_norm_on = bool(fuse_norms)
@@ -200,7 +202,7 @@ class MaskedAttention(Part):
             t[nm["sink"]] = TensorDecl((self.nh,), "bias")
         if self.value_mix is not None:
             # (the source layer's number is part of the checkpoint and is not used)
-            t[nm["vmix"]] = TensorDecl((), "bias", optional=self.value_mix == "source")
+            t[nm["vmix"]] = TensorDecl((), "bias", optional=self.value_mix != "mix")
         return t
 
     def load(self, get: Callable[[str], torch.Tensor], rt: Runtime) -> None:
@@ -237,7 +239,7 @@ class MaskedAttention(Part):
         cos, sin = tables if tables is not None else (None, None)
         q = rt.buffer("mattn.q", (n, nh * d), rt.dtype)
         # the values that layers mix: one buffer per model and step, written by the source layer, read by the others
-        v_first = rt.buffer("mattn.v_first", (n, nkv * dv), torch.float32) if self.value_mix is not None else None
+        v_first = rt.buffer("mattn.v_first", (n, nkv * dv), torch.float32) if self.value_mix in ("source", "mix") else None
         ops.qk_prepare(y, cos, sin, ctx.positions, ctx.tok_entry, cache.block_table, q, cache["k"], cache["v"], nh, nkv,
                        d, dv, self.unit_rms_eps, q_temp=self.q_temp, v_first=v_first, v_lambda=self.v_lambda)
         out = rt.buffer("mattn.out", (n, nh * dv), rt.dtype)
