@@ -86,6 +86,7 @@ def step_parts(runner, mixers, xs, cuts):
     (1, 8, 16, 8, 16, 16, 1, True, False),       # one head that sees itself alone
     (2, 24, 0, 40, 48, 0, 16, True, True),       # nothing rotated
     (2, 16, 32, 8, 320, 32, 50, True, True),     # a low-rank vector wider than the matrix-core kernels take
+    (20, 16, 16, 8, 16, 16, 30, True, True),     # more heads than the 16 rows of a decoding product: two tiles of heads
 ])
 def test_latent_attention_part(dtype, nh, dn, dr, dv, rank, rot, window, sink, gate):
     from vt_transformer_amd.engine.step import ModelRunner
